@@ -44,7 +44,7 @@ typedef void* nvx_stream_t;
  *   8: layers with a 32-bit residual stream and per-sequence state (`nvx_boundary_norm`, `nvx_canon_conv`, `nvx_relu2`,
  *      `nvx_mingru_scan`) and latent attention (`nvx_latent_prep`, `nvx_latent_attn`) added.
  *   9: nvx_boundary_norm can apply the convolution of a decode step in the same launch. */
-#define NVX_ABI_VERSION 15
+#define NVX_ABI_VERSION 16
 
 /* Library identification and diagnostics. */
 int nvx_abi_version(void);
@@ -524,23 +524,40 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  *     head are rotated in pairs (i, i + rot_dims / 2) by the angle positions[t] * freq[i]: (u, v) -> mag * (u cos - v sin, v cos
  *     + u sin).  q_out[t] takes the rotated q, k_cache[slots[t]] the rotated k, v_cache[slots[t]] each value head divided by its
  *     root mean square (with eps).  A negative slot stores nothing.
+ * nvx_attn_prep_store:  q, k, v = heads * dim, kv_heads * dim, kv_heads * vdim elements of x[t] at q_off, k_off, v_off (kv_heads == 0:
+ *     queries only, for a layer that reads another layer's keys and values).  norm_mode 1: every q and k head divided by its root
+ *     mean square, times q_w / k_w (dim entries, shared by the heads); 2: the whole q row and the whole k row likewise (q_w: heads *
+ *     dim, k_w: kv_heads * dim entries); 0: none.  Then the first rot_dims of every q and k head are turned in pairs by positions[t] *
+ *     freq[m], pair m = (m, m + rot_dims / 2) or (2m, 2m + 1) if `interleaved`; with vfreq (vdim / 2 entries) every value head is
+ *     turned over all of vdim by positions[t] * vfreq[m] in the same pair layout.  q_out[t], k_cache[slots[t]], v_cache[slots[t]]
+ *     take the results; a negative slot stores no key or value.
  * nvx_softcap_attn:  token t of sequence b attends over the rows at slots kv_indices[kv_start[b] + j], j <= kv_len[b] - q_len[b] +
- *     (t - qo_indptr[b]):  s_j = scale * q . k_j,  s_j <- cap tanh(s_j / cap) (cap > 0),  out = softmax(s) V.  Query head h reads
+ *     (t - qo_indptr[b]) (and, with window > 0, only the last `window` of them: itself and the window - 1 before it):
+ *     s_j = scale * q . k_j,  s_j <- cap tanh(s_j / cap) (cap > 0),  s_j <- s_j - r1[h] ln(1 + r2[h] (i - j)) (r1, r2 != null; i the
+ *     query's position),  out = softmax(s) V; with vfreq the pairs of out are turned by -i * vfreq[m] (the counterpart of
+ *     nvx_attn_prep_store's rotated values), with gate out is multiplied by sigmoid(gate[t]) (same layout as out).  Query head h reads
  *     key/value head h / (heads / kv_heads).  q (n_tok, heads * dim), k_cache (slots, kv_heads * dim), v_cache (slots, kv_heads *
  *     vdim), out (n_tok, heads * vdim).  n_split > 1 (for steps of few tokens): a (token, head)'s keys are dealt out over n_split
  *     workgroups whose partial results go to `part` (n_tok * heads * n_split * (vdim + 2) floats) and are merged by a second launch.
  * nvx_moe_route:  idx[t][k], wts[t][k] = the expert with the k-th largest logit of token t (ties: the lower id) and the sigmoid
  *     of that logit.
- * Expert e:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + 1), result W_down y, with
- *     w_gu (experts, 2 ff, width) = rows [gate | up] and w_d (experts, width, ff).
- * nvx_moe_expert_rows:  out[t] = sum_k expert_idx[t][k](wts[t][k] * h[t]), the experts' rows streamed per (token, choice) pair by
+ * Expert e:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + shift), result W_down y, with
+ *     w_gu (experts, 2 ff, width) = rows [gate | up] and w_d (experts, width, ff).  (limit = infinity, alpha = 1, shift = 0: silu(g) u.)
+ * nvx_moe_expert_rows:  out[t] = sum_k expert_idx[t][k](wts[t][k] * h[t]), or sum_k wts[t][k] * expert_idx[t][k](h[t]) if
+ *     weight_out; the experts' rows streamed per (token, choice) pair by
  *     workgroups of a few dozen rows; ws: n_tok * top * ff floats (the hidden activations between its two launches); width <=
  *     nvx_moe_expert_rows_max_width(ff).
  * nvx_moe_order:  dst[r] = place of pair r (= token * top + choice) when the n pairs are put in expert order, pairs of one expert
  *     keeping their order; counts[e] = pairs of expert e.  n_exp <= nvx_moe_order_max_experts().
- * nvx_moe_scatter_rows:  xs[dst[r]] = wts[r] * h[r / top] for every (token, choice) pair r.
+ * nvx_moe_scatter_rows:  xs[dst[r]] = wts[r] * h[r / top] for every (token, choice) pair r (wts == null: ones).
  * nvx_moe_glu:  y[r][j] = the expert's activation of (gu[r][j], gu[r][ff + j]).
- * nvx_moe_gather_rows:  out[t] = sum_k ys[dst[t * top + k]].
+ * nvx_moe_gather_rows:  out[t] = sum_k wts[t * top + k] * ys[dst[t * top + k]] (wts == null: ones).
+ * nvx_decay_scan:  x[t] holds q at q_off, k at k_off (heads * dim each) and v at v_off (heads * vdim); act 1: silu of all three first.
+ *     S <- decay[h] S + k v^T;  out[t] = S^T q.   S (slots, heads, dim, vdim), decay (heads) float32.  dim <= 512.
+ * nvx_postnorm_residual:  r = a y[t] (+ b y2[t]);  x[t] += r / rms(r) * w_post (w_post_n = 1: one number, = width: per channel);
+ *     h_out[t] = x[t] / rms(x[t]) * w_next (w_next != null) or x[t] itself, in the format `fmt`.  rms(z) = sqrt(mean z^2 + eps).
+ * nvx_embed_scale:  x[t] = table[ids[t]] * scale (float32), h[t] the same in the table's format (h may be null).
+ * nvx_tanh_cap:  out[i] = cap tanh(in[i] / cap) in float32 (cap <= 0: a copy).
  * nvx_skinny_proj:  out[t][n] = sum_k w[n][k] * f(x[t][k]) in float32, f = identity (in_act 0) or tanh (1); w float32 (n_out,
  *     k_in), x in the format `fmt`.  Meant for few outputs (gate and router logits) or few inputs (the second half of a low-rank
  *     map); one fixed summation order, no workspace. */
@@ -577,19 +594,36 @@ int nvx_rope_vnorm_store(const void* x, int64_t x_stride, int fmt, const int64_t
 int nvx_softcap_attn(const void* q, const void* k_cache, const void* v_cache, int fmt, const int32_t* kv_indices,
                      const int64_t* kv_start, const int32_t* kv_len, const int32_t* qo_indptr, const int32_t* tok_seq,
                      float scale, float cap, void* out, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
-                     int n_split, float* part, nvx_stream_t stream);
+                     int n_split, float* part, int64_t window, const float* r1, const float* r2, const double* vfreq,
+                     int v_interleaved, const void* gate, int64_t gate_stride, nvx_stream_t stream);
+int nvx_attn_prep_store(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off,
+                        const int64_t* positions, const float* q_w, const float* k_w, int norm_mode, float eps, const double* freq,
+                        int rot_dims, int interleaved, const double* vfreq, const int64_t* slots, void* q_out, void* k_cache,
+                        void* v_cache, int64_t n_slots, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
+                        nvx_stream_t stream);
+int nvx_decay_scan(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off, int act,
+                   const float* decay, float* S, int64_t n_slots, const int32_t* qo_indptr, const int64_t* pos0,
+                   const int32_t* state_slot, float* out, int64_t n_tok, int64_t n_seq, int64_t heads, int64_t dim, int64_t vdim,
+                   nvx_stream_t stream);
+int nvx_postnorm_residual(const void* y, int64_t y_stride, const void* y2, int64_t y2_stride, float a, float b, const float* w_post,
+                          int64_t w_post_n, int fmt, float* x, const float* w_next, int64_t w_next_n, float eps, void* h_out,
+                          int64_t n_tok, int64_t width, nvx_stream_t stream);
+int nvx_embed_scale(const int64_t* ids, const void* table, int fmt, int64_t vocab, float scale, float* x, void* h, int64_t n_tok,
+                    int64_t width, nvx_stream_t stream);
+int nvx_tanh_cap(const void* in, int fmt, float cap, float* out, int64_t n, nvx_stream_t stream);
 int nvx_moe_route(const float* logits, int64_t n_tok, int64_t n_exp, int64_t top, int32_t* idx, float* wts, nvx_stream_t stream);
 int64_t nvx_moe_expert_rows_max_width(int64_t ff);
 int nvx_moe_expert_rows(const void* h, int64_t h_stride, int fmt, const int32_t* idx, const float* wts, int64_t top,
-                        const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, float* ws, void* out,
-                        int64_t n_tok, int64_t width, int64_t ff, nvx_stream_t stream);
+                        const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, float shift, int weight_out,
+                        float* ws, void* out, int64_t n_tok, int64_t width, int64_t ff, nvx_stream_t stream);
 int64_t nvx_moe_order_max_experts(void);
 int nvx_moe_order(const int32_t* idx, int64_t n, int64_t n_exp, int64_t* dst, int32_t* counts, nvx_stream_t stream);
 int nvx_moe_scatter_rows(const void* h, int64_t h_stride, int fmt, const float* wts, const int64_t* dst, int64_t top, void* xs,
                          int64_t n_tok, int64_t width, nvx_stream_t stream);
-int nvx_moe_glu(const void* gu, int fmt, float limit, float alpha, void* y, int64_t rows, int64_t ff, nvx_stream_t stream);
-int nvx_moe_gather_rows(const void* ys, int fmt, const int64_t* dst, int64_t top, void* out, int64_t n_tok, int64_t width,
-                        nvx_stream_t stream);
+int nvx_moe_glu(const void* gu, int fmt, float limit, float alpha, float shift, void* y, int64_t rows, int64_t ff,
+                nvx_stream_t stream);
+int nvx_moe_gather_rows(const void* ys, int fmt, const int64_t* dst, const float* wts, int64_t top, void* out, int64_t n_tok,
+                        int64_t width, nvx_stream_t stream);
 int nvx_skinny_proj(const void* x, int64_t x_stride, int fmt, const float* w, int in_act, float* out, int64_t n_tok,
                     int64_t n_out, int64_t k_in, nvx_stream_t stream);
 

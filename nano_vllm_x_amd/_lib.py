@@ -109,16 +109,24 @@ SIGNATURES = {
     "nvx_rope_vnorm_store": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_f32, _c_i32, _c_f32, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64,
                                       _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
     "nvx_softcap_attn": (_c_i32, [_c_vp, _c_vp, _c_vp, _c_i32, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64, _c_i64,
-                                  _c_i64, _c_i64, _c_i32, _c_vp, _c_vp]),
+                                  _c_i64, _c_i64, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_i32, _c_vp, _c_i64, _c_vp]),
+    "nvx_attn_prep_store": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_vp, _c_i32, _c_f32, _c_vp, _c_i32, _c_i32,
+                                     _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
+    "nvx_decay_scan": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_i64, _c_i64, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp,
+                                _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
+    "nvx_postnorm_residual": (_c_i32, [_c_vp, _c_i64, _c_vp, _c_i64, _c_f32, _c_f32, _c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_f32, _c_vp,
+                                       _c_i64, _c_i64, _c_vp]),
+    "nvx_embed_scale": (_c_i32, [_c_vp, _c_vp, _c_i32, _c_i64, _c_f32, _c_vp, _c_vp, _c_i64, _c_i64, _c_vp]),
+    "nvx_tanh_cap": (_c_i32, [_c_vp, _c_i32, _c_f32, _c_vp, _c_i64, _c_vp]),
     "nvx_moe_route": (_c_i32, [_c_vp, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_vp]),
     "nvx_moe_expert_rows_max_width": (_c_i64, [_c_i64]),
-    "nvx_moe_expert_rows": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_i64, _c_f32, _c_f32, _c_vp, _c_vp, _c_i64,
-                                     _c_i64, _c_i64, _c_vp]),
+    "nvx_moe_expert_rows": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_i64, _c_f32, _c_f32, _c_f32, _c_i32, _c_vp,
+                                     _c_vp, _c_i64, _c_i64, _c_i64, _c_vp]),
     "nvx_moe_order_max_experts": (_c_i64, []),
     "nvx_moe_order": (_c_i32, [_c_vp, _c_i64, _c_i64, _c_vp, _c_vp, _c_vp]),
     "nvx_moe_scatter_rows": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp]),
-    "nvx_moe_glu": (_c_i32, [_c_vp, _c_i32, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64, _c_vp]),
-    "nvx_moe_gather_rows": (_c_i32, [_c_vp, _c_i32, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp]),
+    "nvx_moe_glu": (_c_i32, [_c_vp, _c_i32, _c_f32, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64, _c_vp]),
+    "nvx_moe_gather_rows": (_c_i32, [_c_vp, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp]),
     "nvx_skinny_proj": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_i32, _c_vp, _c_i64, _c_i64, _c_i64, _c_vp]),
 }
 

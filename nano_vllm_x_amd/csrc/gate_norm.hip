@@ -2,7 +2,10 @@
 // results pass a learned sigmoid gate before they are added:
 //   - gated residual + grouped RMS norm, one launch per boundary (optionally the result is first formed as the mean of two
 //     RMS-normed branch outputs);
-//   - per-head RMS norm of a recurrence's or attention's read-out, times a weight, times an output gate.
+//   - per-head RMS norm of a recurrence's or attention's read-out, times a weight, times an output gate;
+//   - stacks that norm a sublayer's OUTPUT instead of its input: the (weighted sum of one or two) results divided by its root
+//     mean square, times a weight (one number or one per channel), added to the stream, which the next sublayer reads as it is;
+//   - the two ends of such a stack: scaled embedding rows into the stream, and logits through cap * tanh(. / cap).
 // Norms, gates and the stream are float32 in every activation format.
 #include "fmt_dev.h"
 
@@ -54,6 +57,70 @@ __global__ __launch_bounds__(256) void gated_residual_norm_kernel(
         if (!w_norm) continue;
         const float rn = 1.0f / sqrtf(block256_sum(ss, red) / (float)gs + eps);
         for (int c = lo + threadIdx.x; c < hi; c += 256) st_f(h_out, row + c, x[row + c] * rn * w_norm[c]);   // own stores, read back
+    }
+}
+
+// Per token t (one workgroup):
+//   r = a * y[t] (+ b * y2[t]);  x[t] += r / rms(r) * w_post                  (y != null; w_post: one number or `width` of them)
+//   h[t] = x[t] / rms(x[t]) * w_next  (w_next != null)   or   h[t] = x[t]     (h_out != null)
+template <typename A>
+__global__ __launch_bounds__(256) void postnorm_residual_kernel(const A* __restrict__ y, int64_t y_stride, const A* __restrict__ y2,
+                                                               int64_t y2_stride, float a, float b, const float* __restrict__ w_post,
+                                                               int w_post_n, float* __restrict__ x, const float* __restrict__ w_next,
+                                                               int w_next_n, float eps, A* __restrict__ h_out, int width) {
+    __shared__ float red[4];
+    const int64_t t = blockIdx.x;
+    float* xr = x + t * (int64_t)width;
+    const A* yr = y ? y + t * y_stride : nullptr;
+    const A* y2r = y2 ? y2 + t * y2_stride : nullptr;
+    float rn = 0.f;
+    if (yr) {
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < width; c += 256) {
+            const float r = a * ld_f(yr, c) + (y2r ? b * ld_f(y2r, c) : 0.f);
+            ss += r * r;
+        }
+        rn = 1.0f / sqrtf(block256_sum(ss, red) / (float)width + eps);
+    }
+    float sx = 0.f;
+    for (int c = threadIdx.x; c < width; c += 256) {
+        float xv = xr[c];
+        if (yr) {
+            const float r = a * ld_f(yr, c) + (y2r ? b * ld_f(y2r, c) : 0.f);
+            xv += r * rn * w_post[w_post_n == 1 ? 0 : c];
+            xr[c] = xv;
+        }
+        sx += xv * xv;
+    }
+    if (!h_out) return;
+    A* hr = h_out + t * (int64_t)width;
+    if (w_next) {
+        const float rx = 1.0f / sqrtf(block256_sum(sx, red) / (float)width + eps);
+        for (int c = threadIdx.x; c < width; c += 256) st_f(hr, c, xr[c] * rx * w_next[w_next_n == 1 ? 0 : c]);     // own stores, read back
+    } else {
+        for (int c = threadIdx.x; c < width; c += 256) st_f(hr, c, xr[c]);
+    }
+}
+
+// x[t] = table[ids[t]] * scale (float32), h[t] = the same in the activations' format
+template <typename A>
+__global__ __launch_bounds__(256) void embed_scale_kernel(const int64_t* __restrict__ ids, const A* __restrict__ table, int64_t vocab, float scale,
+                                                         float* __restrict__ x, A* __restrict__ h, int width) {
+    const int64_t t = blockIdx.x;
+    int64_t id = ids[t];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    for (int c = threadIdx.x; c < width; c += 256) {
+        const float v = ld_f(table, id * width + c) * scale;
+        x[t * (int64_t)width + c] = v;
+        if (h) st_f(h, t * (int64_t)width + c, v);
+    }
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void tanh_cap_kernel(const A* __restrict__ in, float cap, float* __restrict__ out, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const float z = ld_f(in, i);
+        out[i] = cap > 0.f ? cap * tanhf(z / cap) : z;
     }
 }
 
@@ -200,4 +267,41 @@ extern "C" int nvx_head_norm_gate(const float* o, const float* w, int w_shared, 
     NVX_FMT_CALL(fmt, hipLaunchKernelGGL(head_norm_gate_kernel<A_>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, (hipStream_t)stream, o, w,
                                          w_shared, (const A_*)gate, gate_stride, kind, eps, (A_*)out, rows, (int)heads, (int)vdim));
     return nvx_check_launch("nvx_head_norm_gate");
+}
+
+extern "C" int nvx_postnorm_residual(const void* y, int64_t y_stride, const void* y2, int64_t y2_stride, float a, float b, const float* w_post,
+                                     int64_t w_post_n, int fmt, float* x, const float* w_next, int64_t w_next_n, float eps, void* h_out,
+                                     int64_t n_tok, int64_t width, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_postnorm_residual: fmt must be 0, 1 or 2");
+    NVX_REQUIRE(n_tok >= 0 && width > 0 && width < (1 << 30), NVX_EINVAL, "nvx_postnorm_residual: bad sizes");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(x && (y || h_out), NVX_EINVAL, "nvx_postnorm_residual: null pointer");
+    NVX_REQUIRE(!y || (y_stride >= width && w_post && (w_post_n == 1 || w_post_n == width)), NVX_EINVAL,
+                "nvx_postnorm_residual: a result needs its norm weight (one number or one per channel)");
+    NVX_REQUIRE(!y2 || (y && y2_stride >= width), NVX_EINVAL, "nvx_postnorm_residual: a second result needs a first");
+    NVX_REQUIRE(!w_next || (h_out && (w_next_n == 1 || w_next_n == width)), NVX_EINVAL, "nvx_postnorm_residual: the closing norm needs an output");
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(postnorm_residual_kernel<A_>, dim3((unsigned)n_tok), dim3(256), 0, (hipStream_t)stream, (const A_*)y,
+                                         y_stride, (const A_*)y2, y2_stride, a, b, w_post, (int)w_post_n, x, w_next, (int)w_next_n, eps, (A_*)h_out,
+                                         (int)width));
+    return nvx_check_launch("nvx_postnorm_residual");
+}
+
+extern "C" int nvx_embed_scale(const int64_t* ids, const void* table, int fmt, int64_t vocab, float scale, float* x, void* h, int64_t n_tok,
+                               int64_t width, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2 && n_tok >= 0 && vocab > 0 && width > 0 && width < (1 << 30), NVX_EINVAL, "nvx_embed_scale: bad arguments");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(ids && table && x, NVX_EINVAL, "nvx_embed_scale: null pointer");
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(embed_scale_kernel<A_>, dim3((unsigned)n_tok), dim3(256), 0, (hipStream_t)stream, ids, (const A_*)table, vocab,
+                                         scale, x, (A_*)h, (int)width));
+    return nvx_check_launch("nvx_embed_scale");
+}
+
+extern "C" int nvx_tanh_cap(const void* in, int fmt, float cap, float* out, int64_t n, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2 && n >= 0, NVX_EINVAL, "nvx_tanh_cap: bad arguments");
+    if (n == 0) return NVX_OK;
+    NVX_REQUIRE(in && out, NVX_EINVAL, "nvx_tanh_cap: null pointer");
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 256 * 64) blocks = 256 * 64;
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(tanh_cap_kernel<A_>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const A_*)in, cap, out, n));
+    return nvx_check_launch("nvx_tanh_cap");
 }

@@ -1,11 +1,13 @@
-// Mixture of small gated feed-forward experts with a sigmoid router whose weight scales the chosen expert's INPUT.
+// Mixture of small gated feed-forward experts; a choice's weight scales the chosen expert's INPUT (sigmoid routers) or its
+// OUTPUT (weight_out: fixed weights from a table).
 //   - nvx_moe_route: the `top` largest router logits of every token -> expert ids and sigmoid scores (float32);
 //   - nvx_moe_expert_rows: a token's experts evaluated row by row of their weights: the form for steps of few tokens, where
 //     every chosen expert's weights have to be streamed once per token anyway;
 //   - nvx_moe_order / nvx_moe_scatter_rows / nvx_moe_glu / nvx_moe_gather_rows: the pieces around per-expert matrix products
 //     for steps of many tokens (the expert order of the (token, choice) pairs and the experts' counts, scaled inputs gathered
 //     into that order, the gated activation, the tokens' results summed back).
-// Expert:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + 1), out = W_down y.
+// Expert:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + shift), out = W_down y
+// (limit = infinity, alpha = 1, shift = 0: silu(g) u).
 #include "fmt_dev.h"
 
 namespace NVX_NS {
@@ -28,10 +30,10 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
     }
 }
 
-__device__ __forceinline__ float glu_act(float g, float u, float limit, float alpha) {
+__device__ __forceinline__ float glu_act(float g, float u, float limit, float alpha, float shift) {
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);
-    return g * sigmoid_f(alpha * g) * (u + 1.0f);
+    return g * sigmoid_f(alpha * g) * (u + shift);
 }
 
 // A token's experts row by row.  w_gu: (experts, 2 * ff, width) rows [gate | up]; w_d: (experts, width, ff).  Two launches, both
@@ -106,12 +108,12 @@ constexpr int MOE_ROWS = 32;      // weight rows per workgroup (8 per wave)
 template <typename A, bool VEC>
 __global__ __launch_bounds__(256) void moe_rows_up_kernel(const A* __restrict__ h, int64_t h_stride, const int32_t* __restrict__ idx,
                                                          const float* __restrict__ wts, int top, const A* __restrict__ w_gu, float limit,
-                                                         float alpha, float* __restrict__ y, int width, int ff) {
+                                                         float alpha, float shift, int weight_out, float* __restrict__ y, int width, int ff) {
     extern __shared__ float sm[];      // the scaled input (width)
     const int64_t t = blockIdx.z;
     const int k = blockIdx.y;
     const int e = idx[t * top + k];
-    const float wt = wts[t * top + k];
+    const float wt = weight_out ? 1.0f : wts[t * top + k];
     for (int c = threadIdx.x; c < width; c += 256) sm[c] = (float)(A)(wt * ld_f(h, t * h_stride + c));
     __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -127,12 +129,13 @@ __global__ __launch_bounds__(256) void moe_rows_up_kernel(const A* __restrict__ 
     for (int i = 0; i < MOE_ROWS / 4; ++i) {
         const int j = blockIdx.x * MOE_ROWS + wave * (MOE_ROWS / 4) + i;
         const float gs = wave_sum(g[i]), us = wave_sum(u[i]);
-        if (lane == 0 && j < ff) y[(t * top + k) * ff + j] = (float)(A)glu_act((float)(A)gs, (float)(A)us, limit, alpha);
+        if (lane == 0 && j < ff) y[(t * top + k) * ff + j] = (float)(A)glu_act((float)(A)gs, (float)(A)us, limit, alpha, shift);
     }
 }
 
 template <typename A, bool VEC>
-__global__ __launch_bounds__(256) void moe_rows_down_kernel(const float* __restrict__ y, const int32_t* __restrict__ idx, int top,
+__global__ __launch_bounds__(256) void moe_rows_down_kernel(const float* __restrict__ y, const int32_t* __restrict__ idx,
+                                                           const float* __restrict__ wts, int top, int weight_out,
                                                            const A* __restrict__ w_d, A* __restrict__ out, int width, int ff) {
     extern __shared__ float sm[];      // one choice's hidden activations (ff)
     const int64_t t = blockIdx.y;
@@ -152,8 +155,9 @@ __global__ __launch_bounds__(256) void moe_rows_down_kernel(const float* __restr
             lane_dot2<A, VEC>(wd + (int64_t)(c < width ? c : width - 1) * ff, wd + (int64_t)(c + 1 < width ? c + 1 : width - 1) * ff, sm, ff, lane,
                               part[i], part[i + 1]);
         }
+        const float wo = weight_out ? wts[t * top + k] : 1.0f;
 #pragma unroll
-        for (int i = 0; i < MOE_ROWS / 4; ++i) o[i] += (float)(A)wave_sum(part[i]);
+        for (int i = 0; i < MOE_ROWS / 4; ++i) o[i] += wo * (float)(A)wave_sum(part[i]);
     }
 #pragma unroll
     for (int i = 0; i < MOE_ROWS / 4; ++i) {
@@ -168,30 +172,30 @@ __global__ __launch_bounds__(256) void moe_scatter_rows_kernel(const A* __restri
                                                               const int64_t* __restrict__ dst, int top, A* __restrict__ xs, int width) {
     const int64_t r = blockIdx.x;
     const int64_t t = r / top;
-    const float wt = wts[r];
+    const float wt = wts ? wts[r] : 1.0f;
     A* o = xs + dst[r] * (int64_t)width;
     for (int c = threadIdx.x; c < width; c += 256) st_f(o, c, wt * ld_f(h, t * h_stride + c));
 }
 
 // y[r][j] = act(gu[r][j], gu[r][ff + j])
 template <typename A>
-__global__ __launch_bounds__(256) void moe_glu_kernel(const A* __restrict__ gu, A* __restrict__ y, float limit, float alpha, int64_t rows,
-                                                     int ff) {
+__global__ __launch_bounds__(256) void moe_glu_kernel(const A* __restrict__ gu, A* __restrict__ y, float limit, float alpha, float shift,
+                                                     int64_t rows, int ff) {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < rows * ff; i += (int64_t)gridDim.x * 256) {
         const int64_t r = i / ff;
         const int j = (int)(i % ff);
-        st_f(y, i, glu_act(ld_f(gu, r * 2 * ff + j), ld_f(gu, r * 2 * ff + ff + j), limit, alpha));
+        st_f(y, i, glu_act(ld_f(gu, r * 2 * ff + j), ld_f(gu, r * 2 * ff + ff + j), limit, alpha, shift));
     }
 }
 
-// out[t] = sum_k ys[dst[t * top + k]]
+// out[t] = sum_k wts[t * top + k] * ys[dst[t * top + k]]   (wts == null: ones)
 template <typename A>
-__global__ __launch_bounds__(256) void moe_gather_rows_kernel(const A* __restrict__ ys, const int64_t* __restrict__ dst, int top,
-                                                             A* __restrict__ out, int width) {
+__global__ __launch_bounds__(256) void moe_gather_rows_kernel(const A* __restrict__ ys, const int64_t* __restrict__ dst,
+                                                             const float* __restrict__ wts, int top, A* __restrict__ out, int width) {
     const int64_t t = blockIdx.x;
     for (int c = threadIdx.x; c < width; c += 256) {
         float o = 0.f;
-        for (int k = 0; k < top; ++k) o += ld_f(ys, dst[t * top + k] * (int64_t)width + c);
+        for (int k = 0; k < top; ++k) o += (wts ? wts[t * top + k] : 1.0f) * ld_f(ys, dst[t * top + k] * (int64_t)width + c);
         st_f(out, t * (int64_t)width + c, o);
     }
 }
@@ -261,33 +265,34 @@ extern "C" int64_t nvx_moe_expert_rows_max_width(int64_t ff) {
 
 template <typename A>
 static void launch_moe_rows(const void* h, int64_t h_stride, const int32_t* idx, const float* wts, int top, const void* w_gu, const void* w_d,
-                            float limit, float alpha, float* ws, void* out, int64_t n_tok, int width, int ff, hipStream_t s) {
+                            float limit, float alpha, float shift, int weight_out, float* ws, void* out, int64_t n_tok, int width, int ff,
+                            hipStream_t s) {
     const bool vec = sizeof(A) == 2 && width % 8 == 0 && ff % 8 == 0 && nvx_aligned16(w_gu) && nvx_aligned16(w_d);
     const dim3 up((unsigned)((ff + MOE_ROWS - 1) / MOE_ROWS), (unsigned)top, (unsigned)n_tok);
     const dim3 down((unsigned)((width + MOE_ROWS - 1) / MOE_ROWS), (unsigned)n_tok);
     if (vec) {
         hipLaunchKernelGGL((moe_rows_up_kernel<A, true>), up, dim3(256), (size_t)width * sizeof(float), s, (const A*)h, h_stride, idx, wts, top,
-                           (const A*)w_gu, limit, alpha, ws, width, ff);
-        hipLaunchKernelGGL((moe_rows_down_kernel<A, true>), down, dim3(256), (size_t)ff * sizeof(float), s, (const float*)ws, idx, top,
-                           (const A*)w_d, (A*)out, width, ff);
+                           (const A*)w_gu, limit, alpha, shift, weight_out, ws, width, ff);
+        hipLaunchKernelGGL((moe_rows_down_kernel<A, true>), down, dim3(256), (size_t)ff * sizeof(float), s, (const float*)ws, idx, wts, top,
+                           weight_out, (const A*)w_d, (A*)out, width, ff);
     } else {
         hipLaunchKernelGGL((moe_rows_up_kernel<A, false>), up, dim3(256), (size_t)width * sizeof(float), s, (const A*)h, h_stride, idx, wts, top,
-                           (const A*)w_gu, limit, alpha, ws, width, ff);
-        hipLaunchKernelGGL((moe_rows_down_kernel<A, false>), down, dim3(256), (size_t)ff * sizeof(float), s, (const float*)ws, idx, top,
-                           (const A*)w_d, (A*)out, width, ff);
+                           (const A*)w_gu, limit, alpha, shift, weight_out, ws, width, ff);
+        hipLaunchKernelGGL((moe_rows_down_kernel<A, false>), down, dim3(256), (size_t)ff * sizeof(float), s, (const float*)ws, idx, wts, top,
+                           weight_out, (const A*)w_d, (A*)out, width, ff);
     }
 }
 
 extern "C" int nvx_moe_expert_rows(const void* h, int64_t h_stride, int fmt, const int32_t* idx, const float* wts, int64_t top,
-                                   const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, float* ws, void* out,
-                                   int64_t n_tok, int64_t width, int64_t ff, nvx_stream_t stream) {
+                                   const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, float shift, int weight_out,
+                                   float* ws, void* out, int64_t n_tok, int64_t width, int64_t ff, nvx_stream_t stream) {
     NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_moe_expert_rows: fmt must be 0, 1 or 2");
     NVX_REQUIRE(n_tok >= 0 && n_tok <= 65535 && top > 0 && top <= 65535 && n_exp > 0 && width > 0 && ff > 0 && h_stride >= width, NVX_EINVAL,
                 "nvx_moe_expert_rows: bad sizes (at most 65535 tokens a step)");
     NVX_REQUIRE(width <= nvx_moe_expert_rows_max_width(ff), NVX_EUNSUPPORTED, "nvx_moe_expert_rows: a row or the hidden size does not fit LDS");
     if (n_tok == 0) return NVX_OK;
     NVX_REQUIRE(h && idx && wts && w_gu && w_d && ws && out, NVX_EINVAL, "nvx_moe_expert_rows: null pointer");
-    NVX_FMT_CALL(fmt, launch_moe_rows<A_>(h, h_stride, idx, wts, (int)top, w_gu, w_d, limit, alpha, ws, out, n_tok, (int)width, (int)ff,
+    NVX_FMT_CALL(fmt, launch_moe_rows<A_>(h, h_stride, idx, wts, (int)top, w_gu, w_d, limit, alpha, shift, weight_out, ws, out, n_tok, (int)width, (int)ff,
                                           (hipStream_t)stream));
     return nvx_check_launch("nvx_moe_expert_rows");
 }
@@ -297,29 +302,30 @@ extern "C" int nvx_moe_scatter_rows(const void* h, int64_t h_stride, int fmt, co
     NVX_REQUIRE(fmt >= 0 && fmt <= 2 && n_tok >= 0 && top > 0 && width > 0 && h_stride >= width && n_tok * top < (1ll << 31), NVX_EINVAL,
                 "nvx_moe_scatter_rows: bad arguments");
     if (n_tok == 0) return NVX_OK;
-    NVX_REQUIRE(h && wts && dst && xs, NVX_EINVAL, "nvx_moe_scatter_rows: null pointer");
+    NVX_REQUIRE(h && dst && xs, NVX_EINVAL, "nvx_moe_scatter_rows: null pointer");
     NVX_FMT_CALL(fmt, hipLaunchKernelGGL(moe_scatter_rows_kernel<A_>, dim3((unsigned)(n_tok * top)), dim3(256), 0, (hipStream_t)stream,
                                          (const A_*)h, h_stride, wts, dst, (int)top, (A_*)xs, (int)width));
     return nvx_check_launch("nvx_moe_scatter_rows");
 }
 
-extern "C" int nvx_moe_glu(const void* gu, int fmt, float limit, float alpha, void* y, int64_t rows, int64_t ff, nvx_stream_t stream) {
+extern "C" int nvx_moe_glu(const void* gu, int fmt, float limit, float alpha, float shift, void* y, int64_t rows, int64_t ff,
+                           nvx_stream_t stream) {
     NVX_REQUIRE(fmt >= 0 && fmt <= 2 && rows >= 0 && ff > 0, NVX_EINVAL, "nvx_moe_glu: bad arguments");
     if (rows == 0) return NVX_OK;
     NVX_REQUIRE(gu && y, NVX_EINVAL, "nvx_moe_glu: null pointer");
     int64_t blocks = (rows * ff + 255) / 256;
     if (blocks > 256 * 64) blocks = 256 * 64;
     NVX_FMT_CALL(fmt, hipLaunchKernelGGL(moe_glu_kernel<A_>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const A_*)gu, (A_*)y, limit,
-                                         alpha, rows, (int)ff));
+                                         alpha, shift, rows, (int)ff));
     return nvx_check_launch("nvx_moe_glu");
 }
 
-extern "C" int nvx_moe_gather_rows(const void* ys, int fmt, const int64_t* dst, int64_t top, void* out, int64_t n_tok, int64_t width,
-                                   nvx_stream_t stream) {
+extern "C" int nvx_moe_gather_rows(const void* ys, int fmt, const int64_t* dst, const float* wts, int64_t top, void* out, int64_t n_tok,
+                                   int64_t width, nvx_stream_t stream) {
     NVX_REQUIRE(fmt >= 0 && fmt <= 2 && n_tok >= 0 && n_tok < (1ll << 31) && top > 0 && width > 0, NVX_EINVAL, "nvx_moe_gather_rows: bad arguments");
     if (n_tok == 0) return NVX_OK;
     NVX_REQUIRE(ys && dst && out, NVX_EINVAL, "nvx_moe_gather_rows: null pointer");
     NVX_FMT_CALL(fmt, hipLaunchKernelGGL(moe_gather_rows_kernel<A_>, dim3((unsigned)n_tok), dim3(256), 0, (hipStream_t)stream, (const A_*)ys, dst,
-                                         (int)top, (A_*)out, (int)width));
+                                         wts, (int)top, (A_*)out, (int)width));
     return nvx_check_launch("nvx_moe_gather_rows");
 }

@@ -4,7 +4,8 @@
 //   - three recurrences over a (key size x value size) memory per head:
 //       mlstm   exponential input gate and sigmoid forget gate stabilised by a running maximum, normaliser vector;
 //       delta   per-head decay, then a rank-one correction of the memory towards the new value along the key;
-//       rwkv    per-key-channel decay, the current token read with a bonus before it is written.
+//       rwkv    per-key-channel decay, the current token read with a bonus before it is written;
+//       decay   one constant decay per head, the token written before it is read (linear attention with a fixed decay).
 // One kernel per recurrence serves prompts, portions of prompts and single decoded tokens: a workgroup takes one head of
 // one sequence and a block of value columns, a thread keeps KR rows of one column in registers, P neighbouring lanes
 // share a column and add their partial read-outs by lane exchange.  The tokens' keys, queries and values are staged
@@ -363,6 +364,71 @@ __global__ __launch_bounds__(256) void rwkv_scan_kernel(const A* __restrict__ rx
     }
 }
 
+// Linear attention with a constant decay per head.  x[t] holds q at q_off, k at k_off (heads * dim each) and v at v_off (heads *
+// vdim), pre-activations if act == 1 (silu is applied to all three as they are staged), values as they are if act == 0.
+//   S <- decay[h] S + k v^T;  o = S^T q  (the read sees the token's own write).          S: (slots, heads, dim, vdim).
+__device__ __forceinline__ float scan_act(float z, int act) { return act == 1 ? z * sigmoid_f(z) : z; }
+template <typename A>
+__global__ __launch_bounds__(256) void decay_scan_kernel(const A* __restrict__ x, int64_t x_stride, int q_off, int k_off, int v_off, int act,
+                                                        const float* __restrict__ decay, float* __restrict__ S,
+                                                        const int32_t* __restrict__ qo_indptr, const int64_t* __restrict__ pos0,
+                                                        const int32_t* __restrict__ state_slot, float* __restrict__ out, int heads, int dim,
+                                                        int vdim, int p_lanes) {
+    extern __shared__ float sm[];
+    const int cb = blockDim.x / p_lanes, rs = p_lanes * KS;
+    float* sq = sm;
+    float* sk = sq + TB * rs;
+    float* sv = sk + TB * rs;
+    const int hd = blockIdx.y;
+    const SeqSpan sp = seq_span(blockIdx.z, qo_indptr, pos0, state_slot);
+    if (sp.slot < 0 || sp.n <= 0) return;
+    const ScanThread th = scan_thread(p_lanes, vdim);
+    float* Sp = S + ((int64_t)sp.slot * heads + hd) * dim * vdim;
+    float s[KR];
+    const bool cont = sp.pos0 > 0;
+#pragma unroll
+    for (int r = 0; r < KR; ++r) {
+        const int row = th.r0 + r;
+        s[r] = (cont && row < dim && th.active) ? Sp[(int64_t)row * vdim + th.e] : 0.f;
+    }
+    zero_rows(sq, 2 * TB * rs);
+    const float g = decay[hd];
+    for (int64_t t0 = 0; t0 < sp.n; t0 += TB) {
+        const int nt = (int)(sp.n - t0 < TB ? sp.n - t0 : TB);
+        __syncthreads();
+        for (int i = threadIdx.x; i < nt * dim; i += blockDim.x) {
+            const int tt = i / dim, d = i % dim;
+            const int64_t r = (sp.q0 + t0 + tt) * x_stride + hd * dim + d;
+            sq[tt * rs + lds_row(d)] = scan_act(ld_f(x, r + q_off), act);
+            sk[tt * rs + lds_row(d)] = scan_act(ld_f(x, r + k_off), act);
+        }
+        for (int i = threadIdx.x; i < nt * cb; i += blockDim.x) {
+            const int tt = i / cb, c = i % cb;
+            const int e = blockIdx.x * cb + c;
+            sv[i] = e < vdim ? scan_act(ld_f(x, (sp.q0 + t0 + tt) * x_stride + v_off + hd * vdim + e), act) : 0.f;
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float v = sv[tt * cb + th.col];
+            const float* kk = sk + tt * rs + th.p * KS;
+            const float* qq = sq + tt * rs + th.p * KS;
+            float o = 0.f;
+#pragma unroll
+            for (int r = 0; r < KR; ++r) {
+                s[r] = g * s[r] + kk[r] * v;
+                o += s[r] * qq[r];
+            }
+            o = lanes_sum(o, p_lanes);
+            if (th.p == 0 && th.active) out[(sp.q0 + t0 + tt) * (int64_t)heads * vdim + (int64_t)hd * vdim + th.e] = o;
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < KR; ++r) {
+        const int row = th.r0 + r;
+        if (row < dim && th.active) Sp[(int64_t)row * vdim + th.e] = s[r];
+    }
+}
+
 // launch geometry of the three recurrences: lanes per column (a power of two), threads per workgroup, value columns per
 // workgroup
 struct ScanLaunch { int p_lanes, threads, cb; };
@@ -490,4 +556,24 @@ extern "C" int nvx_rwkv_scan(const void* r, const void* k, const void* v, int64_
                                          (const A_*)v, rkv_stride, wlog, w0, bonus, S, qo_indptr, pos0, state_slot, out, (int)heads, (int)dim,
                                          g.p_lanes));
     return nvx_check_launch("nvx_rwkv_scan");
+}
+
+extern "C" int nvx_decay_scan(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off, int act,
+                              const float* decay, float* S, int64_t n_slots, const int32_t* qo_indptr, const int64_t* pos0,
+                              const int32_t* state_slot, float* out, int64_t n_tok, int64_t n_seq, int64_t heads, int64_t dim, int64_t vdim,
+                              nvx_stream_t stream) {
+    NVX_LAYOUT_OK("nvx_decay_scan");
+    ScanLaunch g;
+    NVX_REQUIRE(heads > 0 && heads <= 65535 && dim > 0 && vdim > 0 && vdim < (1 << 24) && n_slots >= 0 && (act == 0 || act == 1), NVX_EINVAL,
+                "nvx_decay_scan: bad sizes");
+    NVX_REQUIRE(scan_launch(dim, vdim, &g), NVX_EUNSUPPORTED, "nvx_decay_scan: key size above 512");
+    NVX_REQUIRE(x && decay && S && out, NVX_EINVAL, "nvx_decay_scan: null pointer");
+    NVX_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && x_stride >= q_off + heads * dim && x_stride >= k_off + heads * dim &&
+                    x_stride >= v_off + heads * vdim, NVX_EINVAL, "nvx_decay_scan: q, k or v lies outside a row");
+    const size_t lds = (size_t)(2 * TB * g.p_lanes * KS + TB * g.cb) * sizeof(float);
+    const dim3 grid((unsigned)((vdim + g.cb - 1) / g.cb), (unsigned)heads, (unsigned)n_seq);
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(decay_scan_kernel<A_>, grid, dim3(g.threads), lds, (hipStream_t)stream, (const A_*)x, x_stride, (int)q_off,
+                                         (int)k_off, (int)v_off, act, decay, S, qo_indptr, pos0, state_slot, out, (int)heads, (int)dim, (int)vdim,
+                                         g.p_lanes));
+    return nvx_check_launch("nvx_decay_scan");
 }

@@ -1,5 +1,7 @@
-"""Causal attention with grouped key/value heads, separate key and value sizes, rotary positions on a leading part of each
-head, unit-mean-square values and capped scores, over per-token key and value rows in the token cache."""
+"""Causal attention with grouped key/value heads and separate key and value sizes over per-token key and value rows in the
+token cache: SoftcapAttention (rotary positions on a leading part of each head, unit-mean-square values, capped scores) and
+NormedAttention (query/key RMS norms, optional rotation of keys AND values, window, distance penalty, output gate, borrowed
+keys and values)."""
 from __future__ import annotations
 
 import torch
@@ -43,3 +45,82 @@ class SoftcapAttention(nn.Module):
         o = ops.softcap_attn(q, k_cache, v_cache, md.kv_indices, md.kv_start, md.kv_len, md.layout, self.scale, self.softcap, self.heads,
                              self.kv_heads, self.dim, self.vdim)
         return self.o_proj(o)
+
+
+class NormedAttention(nn.Module):
+    """Softmax attention whose queries and keys pass an RMS norm, with these parts, each optional:
+      qk_norm   "head": every q and k head by its own root mean square, weight (dim) shared by the heads; "row": all heads of a
+                token's q (and of its k) at once, weights of heads * dim and kv_heads * dim entries; "none"
+      rot       {dims, base, interleaved}: the first `dims` of every q and k head turned by position * base^(-2m/dims), pair m being
+                (m, m + dims/2), or (2m, 2m + 1) if interleaved
+      rotate_values   the value of position j is cached turned by j * base^(-2m/vdim) over all of vdim (same pair layout) and a
+                head's read-out at position i is turned back by i, so every value enters in the frame of its distance to i
+      softcap   scores through cap tanh(. / cap);   window   a token sees itself and the window - 1 before it
+      distance_penalty   r1_h ln(1 + r2_h (i - j)) taken off the score (r1, r2: one number per head)
+      out_gate  the concatenated heads times sigmoid(W_g h);   bias   q, k, v projections with biases
+      kv_source (k_name, v_name) of another layer's cache rows: no key/value projections here, that layer's rows are read.
+    The projections q | k | v | g are rows of ONE matrix product: the module's own (`forward`), or a wider one that the caller
+    shares between several mechanisms (`attend`, with the first column of this module's block)."""
+
+    def __init__(self, width: int, heads: int, kv_heads: int, dim: int, vdim: int, scale: float, eps: float, cache_names, qk_norm: str = "head",
+                 rot: dict | None = None, rotate_values: bool = False, softcap=None, window=None, distance_penalty: bool = False,
+                 out_gate: bool = False, bias: bool = False, kv_source=None, own_proj: bool = True):
+        super().__init__()
+        if heads % kv_heads:
+            raise ValueError("query heads must be a multiple of key/value heads")
+        if qk_norm not in ("head", "row", "none"):
+            raise ValueError(f"unknown query/key norm {qk_norm!r}")
+        self.heads, self.kv_heads, self.dim, self.vdim = heads, kv_heads, dim, vdim
+        self.scale, self.softcap, self.eps, self.window = float(scale), float(softcap or 0.0), eps, int(window or 0)
+        self.qk_norm, self.out_gate, self.borrows = qk_norm, out_gate, kv_source is not None
+        self.k_name, self.v_name = kv_source if self.borrows else cache_names
+        self.rot_dims = int(rot["dims"]) if rot else 0
+        self.interleaved = bool(rot and rot.get("interleaved"))
+        if self.rot_dims % 2 or self.rot_dims > dim:
+            raise ValueError("the rotated part of a head must be even and within the head")
+        if rotate_values and (not rot or vdim % 2):
+            raise ValueError("rotated values need a rotation base and an even value size")
+        self.register_buffer("freq", rotary_frequencies(self.rot_dims, rot["base"])[0].to(torch.float64) if self.rot_dims else None, persistent=False)
+        self.register_buffer("vfreq", rotary_frequencies(vdim, rot["base"])[0].to(torch.float64) if rotate_values else None, persistent=False)
+        n_w = {"head": (dim, dim), "row": (heads * dim, kv_heads * dim), "none": (0, 0)}[qk_norm]
+        if n_w[0]:
+            self.q_norm = nn.Parameter(torch.zeros(n_w[0], dtype=torch.float32))
+            if not self.borrows:
+                self.k_norm = nn.Parameter(torch.zeros(n_w[1], dtype=torch.float32))
+        if distance_penalty:
+            self.r1 = nn.Parameter(torch.zeros(heads, dtype=torch.float32))
+            self.r2 = nn.Parameter(torch.zeros(heads, dtype=torch.float32))
+        else:
+            self.r1 = self.r2 = None
+        # columns of this module's block of a projection: q | k | v | g
+        self.q_cols = heads * dim
+        self.k_cols = 0 if self.borrows else kv_heads * dim
+        self.v_cols = 0 if self.borrows else kv_heads * vdim
+        self.g_cols = heads * vdim if out_gate else 0
+        self.proj_rows = self.q_cols + self.k_cols + self.v_cols + self.g_cols
+        self.has_bias = bias
+        if own_proj:
+            self.in_proj = nn.Linear(width, self.proj_rows, bias=bias)
+            if bias:
+                nn.init.zeros_(self.in_proj.bias)      # the gate's rows have no bias: theirs stays zero
+        self.o_proj = nn.Linear(heads * vdim, width, bias=False)
+
+    def cache_rows(self) -> dict:
+        return {} if self.borrows else {self.k_name: self.kv_heads * self.dim, self.v_name: self.kv_heads * self.vdim}
+
+    def attend(self, x: torch.Tensor, col0: int, positions: torch.Tensor, md) -> torch.Tensor:
+        k_cache, v_cache = md.cache.latent(self.k_name), md.cache.latent(self.v_name)
+        k0 = col0 + self.q_cols
+        v0 = k0 + self.k_cols
+        g0 = v0 + self.v_cols
+        own = not self.borrows
+        q = ops.attn_prep_store(x, (col0, k0, v0), positions, getattr(self, "q_norm", None), getattr(self, "k_norm", None), self.qk_norm, self.eps,
+                                self.freq, self.rot_dims, self.interleaved, self.vfreq if own else None, md.out_slots if own else None,
+                                k_cache if own else None, v_cache if own else None, self.heads, self.kv_heads if own else 0, self.dim, self.vdim)
+        o = ops.softcap_attn(q, k_cache, v_cache, md.kv_indices, md.kv_start, md.kv_len, md.layout, self.scale, self.softcap, self.heads,
+                             self.kv_heads, self.dim, self.vdim, window=self.window, r1=self.r1, r2=self.r2, vfreq=self.vfreq,
+                             v_interleaved=self.interleaved, gate=x[:, g0:g0 + self.g_cols] if self.out_gate else None)
+        return self.o_proj(o)
+
+    def forward(self, h: torch.Tensor, positions: torch.Tensor, md) -> torch.Tensor:
+        return self.attend(self.in_proj(h), 0, positions, md)

@@ -1,4 +1,5 @@
-"""Mixture of small gated feed-forward experts behind a sigmoid router."""
+"""Mixtures of small gated feed-forward experts: behind a sigmoid router whose score scales an expert's input, or chosen by a
+table of token ids with fixed weights on the experts' outputs."""
 from __future__ import annotations
 
 import torch
@@ -8,50 +9,79 @@ from torch import nn
 from .. import ops
 
 
-class SigmoidInputMoE(nn.Module):
-    """scores = sigmoid(W_router h) (float32); every token takes the `top` experts with the largest scores, and a score
-    scales its expert's INPUT (no renormalisation): out = sum_e expert_e(score_e * h).  Expert: g = min(W_gate x, limit),
-    u = clamp(W_up x, -limit, limit), W_down (g * sigmoid(alpha * g) * (u + 1)).
+class ExpertBank(nn.Module):
+    """`experts` gated feed-forward layers of one shape, stacked: w_gu (experts, 2 ff, width) = rows gate | up, w_d (experts, width,
+    ff).  Expert: g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), W_down (g sigmoid(alpha g) (u + shift)) -- limit =
+    inf, alpha = 1, shift = 0 is silu(g) u.  `run` evaluates given choices: idx (T, top) int32 expert ids, wts (T, top) float32
+    which scale the experts' inputs, or their outputs if `weight_out`.
 
-    Steps of few tokens (decode steps, which a hipGraph replays: no host decision may depend on the routing) evaluate each
-    token's experts in one launch, streaming the chosen experts' rows.  Steps of many tokens put the scaled inputs into
-    expert order (ops.moe_order: a counting sort, which also gives the per-expert counts) and run one pair of matrix
-    products per expert that received tokens; the counts are the one host read of that path."""
+    Steps of few tokens (decode steps, which a hipGraph replays: no host decision may depend on the choices) evaluate each
+    token's experts in one launch, streaming the chosen experts' rows.  Steps of many tokens put the inputs into expert order
+    (ops.moe_order: a counting sort, which also gives the per-expert counts) and run one pair of matrix products per expert
+    that received tokens; the counts are the one host read of that path."""
 
     ROWS_PATH_TOKENS = 32
 
-    def __init__(self, width: int, experts: int, top: int, ff: int, limit: float, alpha: float):
+    def __init__(self, width: int, experts: int, top: int, ff: int, limit: float, alpha: float, shift: float):
         super().__init__()
-        self.width, self.experts, self.top, self.ff, self.limit, self.alpha = width, experts, top, ff, float(limit), float(alpha)
-        self.router = nn.Parameter(torch.zeros(experts, width, dtype=torch.float32))
+        self.width, self.experts, self.top, self.ff = width, experts, top, ff
+        self.limit, self.alpha, self.shift = float(limit), float(alpha), float(shift)
         self.w_gu = nn.Parameter(torch.empty(experts, 2 * ff, width))      # rows of an expert: gate | up
         self.w_d = nn.Parameter(torch.empty(experts, width, ff))
         self._rows_fit = None
 
-    def forward(self, h: torch.Tensor, decode_step: bool = False) -> torch.Tensor:
+    def run(self, h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, decode_step: bool, weight_out: bool) -> torch.Tensor:
         t = h.shape[0]
-        idx, wts = ops.moe_route(ops.skinny_proj(h, self.router), self.top)
         if self._rows_fit is None:
             self._rows_fit = ops.moe_expert_rows_fits(self.width, self.ff)
             self._order_fit = ops.moe_order_fits(self.experts)      # more experts than the ordering kernel holds: pair by pair
             if not (self._rows_fit or self._order_fit):
                 raise NotImplementedError(f"{self.experts} experts of {self.ff} x {self.width}: neither expert path is built for these sizes")
         if self._rows_fit and (decode_step or t <= self.ROWS_PATH_TOKENS or not self._order_fit):
-            return ops.moe_expert_rows(h, idx, wts, self.w_gu, self.w_d, self.limit, self.alpha)
+            return ops.moe_expert_rows(h, idx, wts, self.w_gu, self.w_d, self.limit, self.alpha, self.shift, weight_out)
         dst, counts = ops.moe_order(idx, self.experts)
         counts = counts.tolist()
-        xs = ops.moe_scatter_rows(h, wts, dst)
+        xs = ops.moe_scatter_rows(h, None if weight_out else wts, dst)
         gu = torch.empty((xs.shape[0], 2 * self.ff), dtype=h.dtype, device=h.device)
         a = 0
         for e, n in enumerate(counts):
             if n:
                 torch.mm(xs[a:a + n], self.w_gu[e].t(), out=gu[a:a + n])
                 a += n
-        y = ops.moe_glu(gu, self.limit, self.alpha)
+        y = ops.moe_glu(gu, self.limit, self.alpha, self.shift)
         ys = torch.empty((xs.shape[0], self.width), dtype=h.dtype, device=h.device)
         a = 0
         for e, n in enumerate(counts):
             if n:
                 torch.mm(y[a:a + n], self.w_d[e].t(), out=ys[a:a + n])
                 a += n
-        return ops.moe_gather_rows(ys, dst)
+        return ops.moe_gather_rows(ys, dst, wts if weight_out else None)
+
+
+class SigmoidInputMoE(ExpertBank):
+    """scores = sigmoid(W_router h) (float32); every token takes the `top` experts with the largest scores, and a score
+    scales its expert's INPUT (no renormalisation): out = sum_e expert_e(score_e * h).  Expert: g = min(W_gate x, limit),
+    u = clamp(W_up x, -limit, limit), W_down (g * sigmoid(alpha * g) * (u + 1))."""
+
+    def __init__(self, width: int, experts: int, top: int, ff: int, limit: float, alpha: float):
+        super().__init__(width, experts, top, ff, limit, alpha, 1.0)
+        self.router = nn.Parameter(torch.zeros(experts, width, dtype=torch.float32))
+
+    def forward(self, h: torch.Tensor, decode_step: bool = False) -> torch.Tensor:
+        idx, wts = ops.moe_route(ops.skinny_proj(h, self.router), self.top)
+        return self.run(h, idx, wts, decode_step, weight_out=False)
+
+
+class TableMoE(ExpertBank):
+    """No router: `table` (vocab, top) int32 names the experts of every token id (the entries of a row differ); each chosen expert
+    weighs 1 / top and the weights apply to the experts' OUTPUTS.  Expert: W_down (silu(W_gate x) * (W_up x))."""
+
+    def __init__(self, width: int, experts: int, top: int, ff: int, vocab: int):
+        super().__init__(width, experts, top, ff, float("inf"), 1.0, 0.0)
+        self.register_buffer("table", torch.zeros(vocab, top, dtype=torch.int32), persistent=False)
+        self.register_buffer("share", torch.full((1, top), 1.0 / top, dtype=torch.float32), persistent=False)
+
+    def forward(self, h: torch.Tensor, input_ids: torch.Tensor, decode_step: bool = False) -> torch.Tensor:
+        idx = self.table.index_select(0, input_ids)
+        wts = self.share.expand(idx.shape[0], self.top).contiguous()
+        return self.run(h, idx, wts, decode_step, weight_out=True)

@@ -132,3 +132,38 @@ class TimeMix(nn.Module):
         o = ops.rwkv_scan(proj[0], proj[1], proj[2], wlog, self.w0, self.bonus, md.cache.state((n, "S")), md.layout, self.heads, self.dim)
         y = ops.head_norm_gate(o, self.norm, self.eps, gate=proj[3], kind="silu")
         return self.o_proj(y)
+
+
+class DecayLinearAttention(nn.Module):
+    """Linear attention with one constant decay per head: q = silu(W_q h), k = silu(W_k h) (heads x dim), v = silu(W_v h) (heads x
+    vdim); per head S <- decay_h S + k v^T, o = S^T q (the read sees the token's own write, no other scale).  The concatenated heads
+    are divided by their common root mean square, times `norm`, times sigmoid(W_g h), then W_o.  State: S (float32), zero at a
+    sequence's start.  The projections q | k | v | g are rows of one matrix product: the module's own (`forward`), or a wider one
+    the caller shares between several mechanisms (`mix`, with the first column of this module's block)."""
+
+    def __init__(self, width: int, heads: int, dim: int, vdim: int, decay, eps: float, state_name, own_proj: bool = True):
+        super().__init__()
+        decay = [float(d) for d in decay]
+        if len(decay) != heads:
+            raise ValueError(f"{heads} heads need {heads} decays, got {len(decay)}")
+        self.heads, self.dim, self.vdim, self.eps, self.state_name = heads, dim, vdim, eps, state_name
+        self.register_buffer("decay", torch.tensor(decay, dtype=torch.float32), persistent=False)
+        self.proj_rows = 2 * heads * dim + 2 * heads * vdim
+        if own_proj:
+            self.in_proj = nn.Linear(width, self.proj_rows, bias=False)
+        self.norm = _f32(heads * vdim)
+        self.o_proj = nn.Linear(heads * vdim, width, bias=False)
+
+    def state_shapes(self) -> dict:
+        return {(self.state_name, "S"): (self.heads, self.dim, self.vdim)}
+
+    def mix(self, x: torch.Tensor, col0: int, md) -> torch.Tensor:
+        hd, he = self.heads * self.dim, self.heads * self.vdim
+        o = ops.decay_scan(x, (col0, col0 + hd, col0 + 2 * hd), self.decay, md.cache.state((self.state_name, "S")), md.layout, self.heads,
+                           self.dim, self.vdim, act="silu")
+        g0 = col0 + 2 * hd + he
+        y = ops.head_norm_gate(o.view(-1, 1, he), self.norm, self.eps, gate=x[:, g0:g0 + he], kind="sigmoid")
+        return self.o_proj(y)
+
+    def forward(self, h: torch.Tensor, md) -> torch.Tensor:
+        return self.mix(self.in_proj(h), 0, md)

@@ -1058,11 +1058,23 @@ SOFTCAP_SPLITS = 4
 
 
 def softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, layout: StepLayout, scale: float, cap: float, heads: int,
-                 kv_heads: int, dim: int, vdim: int, n_split: Optional[int] = None):
+                 kv_heads: int, dim: int, vdim: int, n_split: Optional[int] = None, window: int = 0, r1=None, r2=None, vfreq=None,
+                 v_interleaved: bool = False, gate=None):
     """Causal attention of q (T, heads * dim) over cached rows: sequence b's tokens are at slots kv_indices[kv_start[b] :
     kv_start[b] + kv_len[b]]; scores scale * q . k pass cap * tanh(. / cap) (cap <= 0: not) before the softmax.
-    Returns (T, heads * vdim) in q's format."""
-    _dev(q, k_cache, v_cache, kv_indices, kv_start, kv_len)
+    `window` > 0: a token sees itself and the window - 1 tokens before it.  `r1`, `r2` (heads, float32): r1 ln(1 + r2 (i - j)) is
+    taken off the score of key j for the query at position i.  `vfreq` (vdim / 2, float64): the read-out's pairs ((m, m + vdim / 2),
+    or (2m, 2m + 1) if `v_interleaved`) are turned by -i * vfreq[m], undoing the turn attn_prep_store gave the values.  `gate`
+    (T, heads * vdim): the read-out times sigmoid(gate).  Returns (T, heads * vdim) in q's format."""
+    _dev(q, k_cache, v_cache, kv_indices, kv_start, kv_len, r1, r2, vfreq, gate)
+    _need((r1 is None) == (r2 is None), "softcap_attn: r1 and r2 go together")
+    for a in (r1, r2):
+        if a is not None:
+            _f32c(a, "softcap_attn: r1, r2")
+            _need(a.numel() == heads, "softcap_attn: r1 and r2 have one number per head")
+    _need(vfreq is None or (vfreq.dtype == torch.float64 and vfreq.is_contiguous() and vfreq.numel() == vdim // 2 and vdim % 2 == 0),
+          "softcap_attn: vfreq must be float64 (vdim / 2)")
+    _need(gate is None or (gate.shape == (q.shape[0], heads * vdim) and gate.stride(1) == 1 and gate.dtype == q.dtype), "softcap_attn: gate shape / format")
     t = q.shape[0]
     _need(q.shape == (t, heads * dim) and q.is_contiguous() and t == layout.n_tok, "softcap_attn: q must be contiguous (T, heads * dim)")
     n_slots = k_cache.shape[0]
@@ -1080,7 +1092,118 @@ def softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, layout: Step
     lib = _lib.load()
     _lib.check(lib.nvx_softcap_attn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _fmt(q), _ptr(kv_indices), _ptr(kv_start), _ptr(kv_len),
                                     _ptr(layout.qo_indptr), _ptr(layout.tok_seq), float(scale), float(cap), _ptr(out), t, heads, kv_heads, dim,
-                                    vdim, n_split, _ptr(part), _stream()), "nvx_softcap_attn")
+                                    vdim, n_split, _ptr(part), int(window or 0), _ptr(r1), _ptr(r2), _ptr(vfreq), int(bool(v_interleaved)),
+                                    _ptr(gate), gate.stride(0) if gate is not None else 0, _stream()), "nvx_softcap_attn")
+    return out
+
+
+def attn_prep_store(x, offsets, positions, q_w, k_w, norm_mode: str, eps: float, freq, rot_dims: int, interleaved: bool, vfreq, slots,
+                    k_cache, v_cache, heads: int, kv_heads: int, dim: int, vdim: int):
+    """After a fused projection x (T, columns) holding q, k, v at the three column `offsets`: RMS norm of q and k (`norm_mode`
+    "head": every head by itself, weights q_w / k_w of `dim` entries shared by the heads; "row": all heads of a token at once,
+    weights of heads * dim / kv_heads * dim entries; "none"), rotation of the first rot_dims of every q and k head by positions *
+    freq (float64, rot_dims / 2; pairs (m, m + rot_dims / 2), or (2m, 2m + 1) if `interleaved`), rotation of every value head over
+    all of vdim by positions * vfreq if vfreq is given, keys and values stored at k_cache[slots] / v_cache[slots].  With kv_heads
+    == 0 only the queries are prepared (k_w, slots and the caches may be None).  Returns the queries (T, heads * dim)."""
+    _dev(x, positions, q_w, k_w, freq, vfreq, slots, k_cache, v_cache)
+    t = x.shape[0]
+    _need(x.dim() == 2 and x.stride(1) == 1, "attn_prep_store: x must be (T, columns) with unit inner stride")
+    _need(positions.dtype == torch.int64 and positions.is_contiguous() and positions.numel() == t, "attn_prep_store: positions must be int64 (T)")
+    mode = {"none": 0, "head": 1, "row": 2}[norm_mode]
+    if mode:
+        _f32c(q_w, "attn_prep_store: q_w")
+        _need(q_w.numel() == (dim if mode == 1 else heads * dim), "attn_prep_store: q_w size")
+        if kv_heads:
+            _f32c(k_w, "attn_prep_store: k_w")
+            _need(k_w.numel() == (dim if mode == 1 else kv_heads * dim), "attn_prep_store: k_w size")
+    _need(rot_dims == 0 or (freq.dtype == torch.float64 and freq.is_contiguous() and freq.numel() == rot_dims // 2), "attn_prep_store: freq must be float64 (rot_dims / 2)")
+    _need(vfreq is None or (vfreq.dtype == torch.float64 and vfreq.is_contiguous() and vfreq.numel() == vdim // 2 and vdim % 2 == 0),
+          "attn_prep_store: vfreq must be float64 (vdim / 2)")
+    n_slots = 0
+    if kv_heads:
+        _need(slots.dtype == torch.int64 and slots.is_contiguous() and slots.numel() == t, "attn_prep_store: slots must be int64 (T)")
+        n_slots = k_cache.shape[0]
+        _need(k_cache.dtype == x.dtype and v_cache.dtype == x.dtype and k_cache.is_contiguous() and v_cache.is_contiguous() and
+              k_cache.shape == (n_slots, kv_heads * dim) and v_cache.shape == (n_slots, kv_heads * vdim), "attn_prep_store: cache shapes")
+    q = torch.empty((t, heads * dim), dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_attn_prep_store(_ptr(x), x.stride(0), _fmt(x), offsets[0], offsets[1], offsets[2], _ptr(positions), _ptr(q_w) if mode else None,
+                                       _ptr(k_w) if mode and kv_heads else None, mode, float(eps), _ptr(freq) if rot_dims else None, rot_dims,
+                                       int(bool(interleaved)), _ptr(vfreq), _ptr(slots) if kv_heads else None, _ptr(q),
+                                       _ptr(k_cache) if kv_heads else None, _ptr(v_cache) if kv_heads else None, n_slots, t, heads, kv_heads, dim,
+                                       vdim, _stream()), "nvx_attn_prep_store")
+    return q
+
+
+def decay_scan(x, offsets, decay, mem, layout: StepLayout, heads: int, dim: int, vdim: int, act: str = "none"):
+    """Linear attention with one constant decay per head.  x (T, columns): q, k (heads * dim each) and v (heads * vdim) at the
+    three column `offsets`, passed through `act` ("none" or "silu") first; decay (heads) float32; mem (slots, heads, dim, vdim)
+    float32, continued and written back.  S <- decay S + k v^T, read-out S^T q.  Returns (T, heads, vdim) float32."""
+    _dev(x, decay, mem)
+    _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[0] == layout.n_tok, "decay_scan: x must be (T, columns) with unit inner stride")
+    _f32c(decay, "decay_scan: decay")
+    _f32c(mem, "decay_scan: mem")
+    n_slots = mem.shape[0]
+    _need(decay.numel() == heads and mem.shape == (n_slots, heads, dim, vdim), "decay_scan: shapes")
+    t = x.shape[0]
+    out = torch.empty((t, heads, vdim), dtype=F32, device=x.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_decay_scan(_ptr(x), x.stride(0), _fmt(x), offsets[0], offsets[1], offsets[2], {"none": 0, "silu": 1}[act], _ptr(decay),
+                                  _ptr(mem), n_slots, *_layout_args(layout), _ptr(out), t, layout.n_seq, heads, dim, vdim, _stream()),
+               "nvx_decay_scan")
+    return out
+
+
+def postnorm_residual(x, y=None, w_post=None, eps: float = 0.0, y2=None, a: float = 1.0, b: float = 1.0, w_next=None, out_dtype=None,
+                      want_h: bool = True):
+    """x (T, width) float32, updated in place: x += r / rms(r) * w_post with r = a * y (+ b * y2) and w_post one number or one per
+    channel (float32).  Returns h (T, width) in `out_dtype` (default: y's): x / rms(x) * w_next if w_next is given (one number or
+    one per channel), else x itself; None if not `want_h`."""
+    _dev(x, y, y2, w_post, w_next)
+    _f32c(x, "postnorm_residual: x")
+    _need(x.dim() == 2, "postnorm_residual: x must be (T, width)")
+    t, width = x.shape
+    for name, r in (("y", y), ("y2", y2)):
+        if r is not None:
+            _need(r.shape == (t, width) and r.stride(1) == 1, f"postnorm_residual: {name} must be (T, width) with unit inner stride")
+    _need(y2 is None or (y is not None and y2.dtype == y.dtype), "postnorm_residual: y2 goes with y, in its format")
+    dtype = out_dtype or (y.dtype if y is not None else None)
+    _need(dtype in _FMT and (y is None or y.dtype == dtype), "postnorm_residual: y and the output share one format")
+    for name, w in (("w_post", w_post), ("w_next", w_next)):
+        if w is not None:
+            _f32c(w, "postnorm_residual: " + name)
+            _need(w.numel() in (1, width), f"postnorm_residual: {name} has one entry or one per channel")
+    _need(y is None or w_post is not None, "postnorm_residual: a result needs its norm weight")
+    h = torch.empty((t, width), dtype=dtype, device=x.device) if (want_h or w_next is not None) else None
+    lib = _lib.load()
+    _lib.check(lib.nvx_postnorm_residual(_ptr(y), y.stride(0) if y is not None else 0, _ptr(y2), y2.stride(0) if y2 is not None else 0, float(a),
+                                         float(b), _ptr(w_post), w_post.numel() if w_post is not None else 0, _FMT[dtype], _ptr(x), _ptr(w_next),
+                                         w_next.numel() if w_next is not None else 0, float(eps), _ptr(h), t, width, _stream()),
+               "nvx_postnorm_residual")
+    return h
+
+
+def embed_scale(ids, table, scale: float):
+    """(x, h): x = table[ids] * scale in float32 and the same rows in the table's format."""
+    _dev(ids, table)
+    _need(ids.dtype == torch.int64 and ids.is_contiguous() and ids.dim() == 1, "embed_scale: ids must be int64 (T)")
+    _need(table.dim() == 2 and table.is_contiguous(), "embed_scale: table must be contiguous (vocab, width)")
+    t, width = ids.numel(), table.shape[1]
+    x = torch.empty((t, width), dtype=F32, device=table.device)
+    h = torch.empty((t, width), dtype=table.dtype, device=table.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_embed_scale(_ptr(ids), _ptr(table), _fmt(table), table.shape[0], float(scale), _ptr(x), _ptr(h), t, width, _stream()),
+               "nvx_embed_scale")
+    return x, h
+
+
+def tanh_cap(z, cap: float):
+    """cap * tanh(z / cap) in float32 (cap <= 0: z as float32)."""
+    _dev(z)
+    _need(z.is_contiguous(), "tanh_cap: z must be contiguous")
+    out = torch.empty(z.shape, dtype=F32, device=z.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_tanh_cap(_ptr(z), _fmt(z), float(cap or 0.0), _ptr(out), z.numel(), _stream()), "nvx_tanh_cap")
     return out
 
 
@@ -1107,9 +1230,10 @@ def _moe_weights(w_gu, w_d, what: str):
     return n_exp, ff2 // 2, width
 
 
-def moe_expert_rows(h, idx, wts, w_gu, w_d, limit: float, alpha: float):
-    """out[t] = sum over token t's chosen experts of expert(score * h[t]); w_gu (experts, 2 * ff, width) = gate | up rows, w_d
-    (experts, width, ff).  The chosen experts' rows are streamed per (token, choice) pair: the form for steps of few tokens."""
+def moe_expert_rows(h, idx, wts, w_gu, w_d, limit: float, alpha: float, shift: float = 1.0, weight_out: bool = False):
+    """out[t] = sum over token t's chosen experts of expert(score * h[t]) (or of score * expert(h[t]) if `weight_out`); w_gu
+    (experts, 2 * ff, width) = gate | up rows, w_d (experts, width, ff); activation min(g, limit) sigmoid(alpha min(g, limit))
+    (clamp(u, +-limit) + shift).  The chosen experts' rows are streamed per (token, choice) pair: the form for steps of few tokens."""
     _dev(h, idx, wts, w_gu, w_d)
     n_exp, ff, width = _moe_weights(w_gu, w_d, "moe_expert_rows")
     t, top = idx.shape
@@ -1119,7 +1243,8 @@ def moe_expert_rows(h, idx, wts, w_gu, w_d, limit: float, alpha: float):
     ws = torch.empty((t, top, ff), dtype=F32, device=h.device)      # the hidden activations between the two launches
     lib = _lib.load()
     _lib.check(lib.nvx_moe_expert_rows(_ptr(h), h.stride(0), _fmt(h), _ptr(idx), _ptr(wts), top, _ptr(w_gu), _ptr(w_d), n_exp, float(limit),
-                                       float(alpha), _ptr(ws), _ptr(out), t, width, ff, _stream()), "nvx_moe_expert_rows")
+                                       float(alpha), float(shift), int(bool(weight_out)), _ptr(ws), _ptr(out), t, width, ff, _stream()),
+               "nvx_moe_expert_rows")
     return out
 
 
@@ -1140,11 +1265,12 @@ def moe_order(idx, n_exp: int):
 
 
 def moe_scatter_rows(h, wts, dst):
-    """xs[dst[r]] = wts[r] * h[r // top] for every (token, choice) pair r (dst: int64 (T, top), a permutation)."""
+    """xs[dst[r]] = wts[r] * h[r // top] for every (token, choice) pair r (dst: int64 (T, top), a permutation; wts None: ones)."""
     _dev(h, wts, dst)
-    t, top = wts.shape
-    _need(h.dim() == 2 and h.shape[0] == t and h.stride(1) == 1 and wts.dtype == F32 and wts.is_contiguous(), "moe_scatter_rows: shapes")
-    _need(dst.dtype == torch.int64 and dst.is_contiguous() and dst.shape == wts.shape, "moe_scatter_rows: dst must be int64 (T, top)")
+    t, top = dst.shape
+    _need(h.dim() == 2 and h.shape[0] == t and h.stride(1) == 1, "moe_scatter_rows: shapes")
+    _need(wts is None or (wts.dtype == F32 and wts.is_contiguous() and wts.shape == dst.shape), "moe_scatter_rows: wts must be float32 (T, top)")
+    _need(dst.dtype == torch.int64 and dst.is_contiguous(), "moe_scatter_rows: dst must be int64 (T, top)")
     xs = torch.empty((t * top, h.shape[1]), dtype=h.dtype, device=h.device)
     lib = _lib.load()
     _lib.check(lib.nvx_moe_scatter_rows(_ptr(h), h.stride(0), _fmt(h), _ptr(wts), _ptr(dst), top, _ptr(xs), t, h.shape[1], _stream()),
@@ -1152,24 +1278,27 @@ def moe_scatter_rows(h, wts, dst):
     return xs
 
 
-def moe_glu(gu, limit: float, alpha: float):
-    """gu (rows, 2 * ff) = gate | up pre-activations -> min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, +-limit) + 1)."""
+def moe_glu(gu, limit: float, alpha: float, shift: float = 1.0):
+    """gu (rows, 2 * ff) = gate | up pre-activations -> min(g, limit) * sigmoid(alpha * min(g, limit)) * (clamp(u, +-limit) + shift)
+    (limit = inf, alpha = 1, shift = 0: silu(g) * u)."""
     _dev(gu)
     _need(gu.dim() == 2 and gu.is_contiguous() and gu.shape[1] % 2 == 0, "moe_glu: gu must be contiguous (rows, 2 * ff)")
     y = torch.empty((gu.shape[0], gu.shape[1] // 2), dtype=gu.dtype, device=gu.device)
     lib = _lib.load()
-    _lib.check(lib.nvx_moe_glu(_ptr(gu), _fmt(gu), float(limit), float(alpha), _ptr(y), gu.shape[0], gu.shape[1] // 2, _stream()), "nvx_moe_glu")
+    _lib.check(lib.nvx_moe_glu(_ptr(gu), _fmt(gu), float(limit), float(alpha), float(shift), _ptr(y), gu.shape[0], gu.shape[1] // 2, _stream()),
+               "nvx_moe_glu")
     return y
 
 
-def moe_gather_rows(ys, dst):
-    """out[t] = sum_k ys[dst[t][k]]."""
-    _dev(ys, dst)
+def moe_gather_rows(ys, dst, wts=None):
+    """out[t] = sum_k wts[t][k] * ys[dst[t][k]] (wts None: ones)."""
+    _dev(ys, dst, wts)
+    _need(wts is None or (wts.dtype == F32 and wts.is_contiguous() and wts.shape == dst.shape), "moe_gather_rows: wts must be float32 (T, top)")
     t, top = dst.shape
     _need(ys.dim() == 2 and ys.is_contiguous() and ys.shape[0] == t * top and dst.dtype == torch.int64 and dst.is_contiguous(), "moe_gather_rows: shapes")
     out = torch.empty((t, ys.shape[1]), dtype=ys.dtype, device=ys.device)
     lib = _lib.load()
-    _lib.check(lib.nvx_moe_gather_rows(_ptr(ys), _fmt(ys), _ptr(dst), top, _ptr(out), t, ys.shape[1], _stream()), "nvx_moe_gather_rows")
+    _lib.check(lib.nvx_moe_gather_rows(_ptr(ys), _fmt(ys), _ptr(dst), _ptr(wts), top, _ptr(out), t, ys.shape[1], _stream()), "nvx_moe_gather_rows")
     return out
 
 

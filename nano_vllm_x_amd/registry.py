@@ -24,8 +24,13 @@ def _meronex():
     return MeronexConfig.from_dict, MeronexForCausalLM
 
 
+def _gibavik():
+    from .gibavik import GibavikConfig, GibavikForCausalLM
+    return GibavikConfig.from_dict, GibavikForCausalLM
+
+
 # architecture name (config.json "architectures"[0] or "architecture") -> loader of (config reader, model class)
-ARCHITECTURES = {"Qwen3ForCausalLM": _qwen3, "Kabidra": _kabidra, "Meronex": _meronex}
+ARCHITECTURES = {"Qwen3ForCausalLM": _qwen3, "Kabidra": _kabidra, "Meronex": _meronex, "Gibavik": _gibavik}
 
 
 def architecture_of(config: dict) -> str:
