@@ -83,13 +83,24 @@ _DEFS = {
     "rope_vnorm_store": "(Tensor qkv, Tensor positions, Tensor? freq, float mag, int rot_dims, float eps, Tensor slots, Tensor(a!) k_cache, "
                         "Tensor(b!) v_cache, int heads, int kv_heads, int dim, int vdim) -> Tensor",
     "softcap_attn": "(Tensor q, Tensor k_cache, Tensor v_cache, Tensor kv_indices, Tensor kv_start, Tensor kv_len, Tensor pos0, "
-                    "Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq, float scale, float cap, int heads, int kv_heads, int dim, int vdim) -> Tensor",
+                    "Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq, float scale, float cap, int heads, int kv_heads, int dim, int vdim, "
+                    "int window=0, Tensor? r1=None, Tensor? r2=None, Tensor? vfreq=None, bool v_interleaved=False, Tensor? gate=None) -> Tensor",
+    # post-normed stream, query/key norms with rotated values, decayed linear attention, experts with weights on their outputs
+    "attn_prep_store": "(Tensor x, int q_off, int k_off, int v_off, Tensor positions, Tensor? q_w, Tensor? k_w, str norm_mode, float eps, "
+                       "Tensor? freq, int rot_dims, bool interleaved, Tensor? vfreq, Tensor? slots, Tensor(a!)? k_cache, Tensor(b!)? v_cache, "
+                       "int heads, int kv_heads, int dim, int vdim) -> Tensor",
+    "decay_scan": "(Tensor x, int q_off, int k_off, int v_off, Tensor decay, Tensor(a!) mem, Tensor pos0, Tensor state_slot, Tensor? qo_indptr, "
+                  "Tensor? tok_seq, int heads, int dim, int vdim, str act) -> Tensor",
+    "postnorm_residual": "(Tensor(a!) x, Tensor? y, Tensor? w_post, float eps, Tensor? y2, float a, float b, Tensor? w_next, ScalarType dtype) -> Tensor",
+    "embed_scale": "(Tensor ids, Tensor table, float scale) -> (Tensor, Tensor)",
+    "tanh_cap": "(Tensor z, float cap) -> Tensor",
     "moe_route": "(Tensor logits, int top) -> (Tensor, Tensor)",
-    "moe_expert_rows": "(Tensor h, Tensor idx, Tensor wts, Tensor w_gu, Tensor w_d, float limit, float alpha) -> Tensor",
+    "moe_expert_rows": "(Tensor h, Tensor idx, Tensor wts, Tensor w_gu, Tensor w_d, float limit, float alpha, float shift=1.0, "
+                       "bool weight_out=False) -> Tensor",
     "moe_order": "(Tensor idx, int n_exp) -> (Tensor, Tensor)",
-    "moe_scatter_rows": "(Tensor h, Tensor wts, Tensor dst) -> Tensor",
-    "moe_glu": "(Tensor gu, float limit, float alpha) -> Tensor",
-    "moe_gather_rows": "(Tensor ys, Tensor dst) -> Tensor",
+    "moe_scatter_rows": "(Tensor h, Tensor? wts, Tensor dst) -> Tensor",
+    "moe_glu": "(Tensor gu, float limit, float alpha, float shift=1.0) -> Tensor",
+    "moe_gather_rows": "(Tensor ys, Tensor dst, Tensor? wts=None) -> Tensor",
     "skinny_proj": "(Tensor x, Tensor w, str in_act) -> Tensor",
 }
 for _name, _sig in _DEFS.items():
@@ -284,17 +295,40 @@ def _rope_vnorm_store(qkv, positions, freq, mag, rot_dims, eps, slots, k_cache, 
     return ops.rope_vnorm_store(qkv, positions, freq, mag, rot_dims, eps, slots, k_cache, v_cache, heads, kv_heads, dim, vdim)
 
 
-def _softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, pos0, state_slot, qo_indptr, tok_seq, scale, cap, heads, kv_heads, dim, vdim):
+def _softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, pos0, state_slot, qo_indptr, tok_seq, scale, cap, heads, kv_heads, dim, vdim,
+                  window=0, r1=None, r2=None, vfreq=None, v_interleaved=False, gate=None):
     return ops.softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, _layout(q.shape[0], pos0, state_slot, qo_indptr, tok_seq), scale, cap,
-                            heads, kv_heads, dim, vdim)
+                            heads, kv_heads, dim, vdim, window=window, r1=r1, r2=r2, vfreq=vfreq, v_interleaved=v_interleaved, gate=gate)
+
+
+def _attn_prep_store(x, q_off, k_off, v_off, positions, q_w, k_w, norm_mode, eps, freq, rot_dims, interleaved, vfreq, slots, k_cache, v_cache,
+                     heads, kv_heads, dim, vdim):
+    return ops.attn_prep_store(x, (q_off, k_off, v_off), positions, q_w, k_w, norm_mode, eps, freq, rot_dims, interleaved, vfreq, slots, k_cache,
+                               v_cache, heads, kv_heads, dim, vdim)
+
+
+def _decay_scan(x, q_off, k_off, v_off, decay, mem, pos0, state_slot, qo_indptr, tok_seq, heads, dim, vdim, act):
+    return ops.decay_scan(x, (q_off, k_off, v_off), decay, mem, _layout(x.shape[0], pos0, state_slot, qo_indptr, tok_seq), heads, dim, vdim, act=act)
+
+
+def _postnorm_residual(x, y, w_post, eps, y2, a, b, w_next, dtype):
+    return ops.postnorm_residual(x, y=y, w_post=w_post, eps=eps, y2=y2, a=a, b=b, w_next=w_next, out_dtype=dtype)
+
+
+def _embed_scale(ids, table, scale):
+    return ops.embed_scale(ids, table, scale)
+
+
+def _tanh_cap(z, cap):
+    return ops.tanh_cap(z, cap)
 
 
 def _moe_route(logits, top):
     return ops.moe_route(logits, top)
 
 
-def _moe_expert_rows(h, idx, wts, w_gu, w_d, limit, alpha):
-    return ops.moe_expert_rows(h, idx, wts, w_gu, w_d, limit, alpha)
+def _moe_expert_rows(h, idx, wts, w_gu, w_d, limit, alpha, shift=1.0, weight_out=False):
+    return ops.moe_expert_rows(h, idx, wts, w_gu, w_d, limit, alpha, shift, weight_out)
 
 
 def _moe_order(idx, n_exp):
@@ -305,12 +339,12 @@ def _moe_scatter_rows(h, wts, dst):
     return ops.moe_scatter_rows(h, wts, dst)
 
 
-def _moe_glu(gu, limit, alpha):
-    return ops.moe_glu(gu, limit, alpha)
+def _moe_glu(gu, limit, alpha, shift=1.0):
+    return ops.moe_glu(gu, limit, alpha, shift)
 
 
-def _moe_gather_rows(ys, dst):
-    return ops.moe_gather_rows(ys, dst)
+def _moe_gather_rows(ys, dst, wts=None):
+    return ops.moe_gather_rows(ys, dst, wts)
 
 
 def _skinny_proj(x, w, in_act):
