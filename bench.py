@@ -642,9 +642,171 @@ def _meronex_kernel_table(z, t_pre, n_dec, ctx, phases=("prefill", "decode")):
             add("moe_expert_rows", phase, us, bytes_=min(t * 2, 8) * 3 * ff * w * 2, like="(library products of the dense feed-forward)")
     return rows
 
+def _gibavik_config(z):
+    """Layers parallel, attention in turn (the last attention layer of six borrows the keys and values of the one before it); heads of
+    128; a window of 512 keys, rotation of 64 dimensions; linear-attention heads with keys 64 and values 128 wide; the first layer's
+    feed-forward dense, the others eight experts of ff / 2 of which a token takes two, so that a token's feed-forward work equals the
+    dense model's."""
+    w, hd = z["width"], z["width"] // 128
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 2}, "router": {"experts": 8, "top": 2}}
+    dense = {"kind": "dense", "ff": z["ff"], "limit": 7.0}
+    par = {"type": "parallel", "mixer": {
+        "left": {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0, "mask": {"size": 512},
+                 "rot": {"dims": 64, "base": 1e6}},
+        "right": {"heads": hd, "dim": 64, "vdim": 128, "decay": [1.0 - 2.0 ** -(3 + j % 8) for j in range(hd)]}, "left_scale": 0.6, "right_scale": 1.1}}
+    att = {"type": "attention", "mixer": {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5}}
+    layers = []
+    for i in range(z["layers"]):
+        layer = json.loads(json.dumps(par if i % 2 == 0 else att))
+        layer["mlp"] = dense if i == 0 else moe
+        if i == 5:
+            layer["mixer"]["kv_from"] = 3
+        layers.append(layer)
+    return {"architecture": "Gibavik", "vocab": z["vocab"], "width": w, "norm": {"eps": 1e-5}, "embedding": {"scale": 8.0}, "logit_softcap": 30.0,
+            "layers": layers}
+
+
+def _gibavik_kernel_table(z, t_pre, n_dec, ctx, phases=("prefill", "decode")):
+    """Each kernel of Gibavik beside the like kernel of Qwen3 (and, at decode shapes, of Meronex) at the same shape: time, and the
+    fraction of its roofline (HBM bytes it must move at 8 TB/s; attention in prefill: its multiply-adds at the dense bf16 MFMA peak;
+    the recurrence in prefill: its multiply-adds at the float32 vector peak, since its state is float32)."""
+    from nano_vllm_x_amd import ops
+    from nano_vllm_x_amd.layers.rotary_embedding import rotary_frequencies
+    dev, bf = torch.device("cuda"), torch.bfloat16
+    w, ff, h = z["width"], z["ff"] // 2, z["heads"]
+    hd, window = w // 128, 512
+    rows = []
+
+    def layout(n_seq, q_len, pos0):
+        p = torch.full((n_seq,), pos0, dtype=torch.int64, device=dev)
+        sl = torch.arange(n_seq, dtype=torch.int32, device=dev)
+        if q_len == 1:
+            return ops.StepLayout(n_seq, n_seq, p, sl)
+        qo = torch.arange(0, n_seq + 1, dtype=torch.int32, device=dev) * q_len
+        return ops.StepLayout(n_seq * q_len, n_seq, p, sl, qo, torch.arange(n_seq, dtype=torch.int32, device=dev).repeat_interleave(q_len))
+
+    def add(name, phase, us, bytes_=None, flops=None, like=None, peak=None):
+        if bytes_:
+            frac, bound = bytes_ / (us * 1e-6) / (HBM_PEAK_GBS * 1e9), "HBM"
+        else:
+            frac, bound = flops / (us * 1e-6) / ((peak or MFMA_BF16_PEAK_TFLOPS) * 1e12), "MFMA" if peak is None else "fp32 VALU"
+        rows.append({"kernel": name, "phase": phase, "us": round(us, 1), "of_roofline": round(frac, 3), "bound": bound, "like": like})
+
+    for phase, (n_seq, q_len, pos0) in (("prefill", (max(t_pre // 1024, 1), 1024, 0)), ("decode", (n_dec, 1, ctx))):
+        if phase not in phases:
+            continue
+        t = n_seq * q_len
+        dec = phase == "decode"
+        lay = layout(n_seq, q_len, pos0)
+        reps = 20 if dec else 3
+        y, y2, x = torch.randn(t, w, device=dev).to(bf), torch.randn(t, w, device=dev).to(bf), torch.randn(t, w, device=dev)
+        one, wv = torch.ones(1, device=dev), torch.ones(w, device=dev)
+        # sublayer boundary: reads the result (2 B; two of them after a parallel mixer) and the stream (4 B), writes the stream (4 B) and
+        # the rows the next sublayer reads (2 B)
+        add("postnorm_residual", phase, _time_us(lambda: ops.postnorm_residual(x, y=y, w_post=one, eps=1e-5)), bytes_=t * w * 12, like="rmsnorm+residual")
+        add("postnorm_residual, two results", phase, _time_us(lambda: ops.postnorm_residual(x, y=y, y2=y2, a=0.6, b=1.1, w_post=one, eps=1e-5)),
+            bytes_=t * w * 14, like="gated_residual_norm")
+        xb = x.to(bf)
+        add("qwen3 rmsnorm+residual", phase, _time_us(lambda: ops.rmsnorm(y, wv.to(bf), 1e-5, xb)), bytes_=t * w * 8)
+        if dec:
+            add("meronex gated_residual_norm", phase, _time_us(lambda: ops.gated_residual_norm(x, y=y, gate=y2, gate_bias=wv, mult=0.5, w_norm=wv, groups=4,
+                                                                                              eps=1e-5)), bytes_=t * w * 14)
+        o32 = torch.randn(t, hd, 128, device=dev)
+        gate = torch.randn(t, w, device=dev).to(bf)
+        add("head_norm_gate, heads normed together", phase, _time_us(lambda: ops.head_norm_gate(o32.view(t, 1, w), wv, 1e-5, gate=gate, kind="sigmoid")),
+            bytes_=t * w * 8, like="head_norm_gate")
+        add("meronex head_norm_gate (head by head)", phase, _time_us(lambda: ops.head_norm_gate(o32, wv, 1e-5, gate=gate, kind="silu")), bytes_=t * w * 8)
+        gu = torch.randn(t, 2 * ff, device=dev).to(bf)
+        add("moe_glu (silu(g) u)", phase, _time_us(lambda: ops.moe_glu(gu, float("inf"), 1.0, 0.0)), bytes_=t * ff * 6, like="silu_mul")
+        add("qwen3 silu_mul", phase, _time_us(lambda: ops.silu_mul(gu)), bytes_=t * ff * 6)
+        # linear attention with a constant decay: keys 64, values 128 wide
+        xr = torch.randn(t, 2 * hd * 64 + 2 * w, device=dev).to(bf)
+        mem = torch.zeros(n_seq + 1, hd, 64, 128, device=dev)
+        decay = torch.full((hd,), 0.99, device=dev)
+        us = _time_us(lambda: ops.decay_scan(xr, (0, hd * 64, 2 * hd * 64), decay, mem, lay, hd, 64, 128, act="silu"), reps)
+        if dec:
+            add("decay_scan", phase, us, bytes_=n_seq * hd * 64 * 128 * 8 + t * (2 * hd * 64 + w) * 2, like="rwkv_scan")
+            h64 = w // 64
+            rkv = torch.randn(3, t, w, device=dev).to(bf)
+            wlog = torch.randn(t, w, device=dev) - 3.0
+            mem3 = torch.zeros(n_seq + 1, h64, 64, 64, device=dev)
+            w0, bonus = torch.zeros(w, device=dev), torch.zeros(h64, 64, device=dev)
+            add("meronex rwkv_scan", phase, _time_us(lambda: ops.rwkv_scan(rkv[0], rkv[1], rkv[2], wlog, w0, bonus, mem3, lay, h64, 64)),
+                bytes_=n_seq * h64 * 64 * 64 * 8 + t * w * 10)
+        else:
+            add("decay_scan", phase, us, flops=4.0 * t * hd * 64 * 128, peak=FP32_VALU_PEAK_TFLOPS, like="mingru_scan")
+        zxg = torch.randn(t, 3 * w, device=dev).to(bf)
+        gs = torch.zeros(n_seq + 1, w, device=dev)
+        add("kabidra mingru_scan", phase, _time_us(lambda: ops.mingru_scan(zxg, gs, lay)), bytes_=t * w * 8 + n_seq * w * 8)
+        # attention: 8 key/value heads of 128, beside paged attention over the same tokens
+        kv_len = pos0 + q_len
+        n_rows = n_seq * kv_len
+        kc, vc = torch.randn(n_rows, 8 * 128, device=dev).to(bf), torch.randn(n_rows, 8 * 128, device=dev).to(bf)
+        idx = torch.arange(n_rows, dtype=torch.int32, device=dev)
+        kv_start = torch.arange(n_seq, dtype=torch.int64, device=dev) * kv_len
+        kvl = torch.full((n_seq,), kv_len, dtype=torch.int32, device=dev)
+        qkv = torch.randn(t, (h + 16) * 128 + h * 128, device=dev).to(bf)          # q | k | v | g
+        pos = (torch.arange(t, device=dev) % q_len + pos0).to(torch.int64)
+        slots = (torch.arange(t, device=dev) // q_len * kv_len + pos).to(torch.int64)
+        fr, vfr = rotary_frequencies(64, 1e6)[0].to(dev), rotary_frequencies(128, 1e6)[0].to(dev)
+        qn = torch.ones(128, device=dev)
+        prep_bytes = t * (h + 16) * 128 * 2 * 2
+        add("attn_prep_store (head norms, rotation, rotated values)", phase,
+            _time_us(lambda: ops.attn_prep_store(qkv, (0, h * 128, (h + 8) * 128), pos, qn, qn, "head", 1e-5, fr, 64, False, vfr, slots, kc, vc, h, 8, 128, 128)),
+            bytes_=prep_bytes, like="rope_vnorm_store / qknorm_rope_store")
+        qr, kr = torch.ones(h * 128, device=dev), torch.ones(8 * 128, device=dev)
+        add("attn_prep_store (row norms)", phase,
+            _time_us(lambda: ops.attn_prep_store(qkv, (0, h * 128, (h + 8) * 128), pos, qr, kr, "row", 1e-5, None, 0, False, None, slots, kc, vc, h, 8, 128, 128)),
+            bytes_=prep_bytes, like="rope_vnorm_store / qknorm_rope_store")
+        if dec:
+            from nano_vllm_x_amd.layers.rotary_embedding import rotary_frequencies as rf
+            fr2, mag = rf(64, 1e6, {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0})
+            fr2 = fr2.to(dev)
+            add("meronex rope_vnorm_store", phase, _time_us(lambda: ops.rope_vnorm_store(qkv[:, :(h + 16) * 128], pos, fr2, mag, 64, 1e-5, slots, kc, vc, h, 8,
+                                                                                        128, 128)), bytes_=prep_bytes)
+        q128 = torch.randn(t, h * 128, device=dev).to(bf)
+        g128 = qkv[:, (h + 16) * 128:]
+        r1, r2 = torch.full((h,), 0.5, device=dev), torch.full((h,), 0.1, device=dev)
+        us_win = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 50.0, h, 8, 128, 128, window=window, vfreq=vfr, gate=g128), reps)
+        us_pen = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 0.0, h, 8, 128, 128, r1=r1, r2=r2), reps)
+        us_plain = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 30.0, h, 8, 128, 128), reps)
+        kc4, vc4 = kc.view(n_rows, 8, 128), vc.view(n_rows, 8, 128)
+        if not dec:
+            pairs = n_seq * q_len * (q_len + 1) // 2
+            pairs_win = n_seq * sum(min(i + 1, window) for i in range(q_len))
+            add("softcap_attn (window, read-out turned back, gate)", phase, us_win, flops=4.0 * h * 128 * pairs_win, like="paged_prefill")
+            add("softcap_attn (distance penalty)", phase, us_pen, flops=4.0 * h * 128 * pairs, like="paged_prefill")
+            add("meronex softcap_attn (capped scores only)", phase, us_plain, flops=4.0 * h * 128 * pairs)
+            plan = ops.prefill_plan_ws(n_seq, dev)
+            kv_indptr = torch.arange(0, n_seq + 1, dtype=torch.int32, device=dev) * kv_len
+            ops.prefill_plan(lay.qo_indptr, plan)
+            us = _time_us(lambda: ops.paged_prefill(q128, kc4, vc4, lay.qo_indptr, kv_indptr, idx, plan, h, 8, 0.1), reps=5)
+            add("qwen3 paged_prefill", phase, us, flops=4.0 * h * 128 * pairs)
+        else:
+            io = 2 * t * h * 128 * 2
+            add("softcap_attn (window, read-out turned back, gate)", phase, us_win, bytes_=n_seq * min(kv_len, window) * 8 * 128 * 2 * 2 + io + t * h * 128 * 2,
+                like="paged_decode")
+            add("softcap_attn (distance penalty)", phase, us_pen, bytes_=n_rows * 8 * 128 * 2 * 2 + io, like="paged_decode")
+            add("meronex softcap_attn (capped scores only)", phase, us_plain, bytes_=n_rows * 8 * 128 * 2 * 2 + io)
+            ws = ops.DecodeWorkspace(n_seq, h, 8, dev)
+            ops.decode_plan(kvl, kv_start, ws)
+            us = _time_us(lambda: ops.paged_decode(q128, kc4, vc4, idx, n_seq, ws, 0.1))
+            add("qwen3 paged_decode", phase, us, bytes_=n_rows * 8 * 128 * 2 * 2 + io)
+            # experts: eight of ff / 2, two a token, the weights on the outputs
+            hm = torch.randn(t, w, device=dev).to(bf)
+            w_gu, w_d = torch.randn(8, 2 * ff, w, device=dev).to(bf) * 0.02, torch.randn(8, w, ff, device=dev).to(bf) * 0.02
+            eidx = torch.stack([torch.randperm(8, device=dev)[:2] for _ in range(t)]).to(torch.int32)
+            wts = torch.full((t, 2), 0.5, device=dev)
+            us = _time_us(lambda: ops.moe_expert_rows(hm, eidx, wts, w_gu, w_d, float("inf"), 1.0, 0.0, True))
+            add("moe_expert_rows (weights on outputs)", phase, us, bytes_=min(t * 2, 8) * 3 * ff * w * 2, like="meronex moe_expert_rows")
+            us = _time_us(lambda: ops.moe_expert_rows(hm, eidx, wts, w_gu, w_d, 7.0, 1.702))
+            add("meronex moe_expert_rows", phase, us, bytes_=min(t * 2, 8) * 3 * ff * w * 2)
+    return rows
+
 
 ARCHS = {"kabidra": (lambda z: _kabidra_config(z), lambda *a, **k: _kernel_table(*a), "Kabidra"),
-         "meronex": (lambda z: _meronex_config(z), lambda *a, **k: _meronex_kernel_table(*a, **k), "Meronex")}
+         "meronex": (lambda z: _meronex_config(z), lambda *a, **k: _meronex_kernel_table(*a, **k), "Meronex"),
+         "gibavik": (lambda z: _gibavik_config(z), lambda *a, **k: _gibavik_kernel_table(*a, **k), "Gibavik")}
 
 
 def arch_compare(args):
@@ -654,7 +816,8 @@ def arch_compare(args):
     make_config, kernel_table, title = ARCHS[args.arch]
     result = {"metric": f"prefill and decode tokens/s, {title} beside Qwen3 at equal width, depth, feed-forward and vocabulary",
               "dtype": "bf16", "data": "synthetic (random token ids, random-init weights)", "n_gpus": 1,
-              "workload": {"prefill": f"{args.arch_seqs} prompts of {args.arch_prompt} tokens in one step",
+              "workload": {"prefill": f"{args.arch_seqs} prompts of {args.arch_prompt} tokens in " +
+                                      (f"steps of at most {args.arch_portion} tokens" if args.arch_portion else "one step"),
                            "decode": f"{args.arch_seqs} sequences, {args.arch_new} steps from context {args.arch_prompt}"},
               "sizes": {}}
     if args.arch == "meronex" and args.arch_serve and not args.arch_portion:
@@ -678,7 +841,10 @@ def arch_compare(args):
             continue
         print(f"[arch-compare] {name}: kernels one by one", file=sys.stderr, flush=True)
         with torch.inference_mode():
-            entry["kernels"] = kernel_table(z, args.arch_seqs * args.arch_prompt, args.arch_seqs, args.arch_prompt,
+            t_pre = args.arch_seqs * args.arch_prompt
+            if args.arch == "gibavik" and args.arch_portion:      # the kernels one by one at the size of the steps the engines ran
+                t_pre = min(t_pre, max(args.arch_portion, args.arch_prompt))
+            entry["kernels"] = kernel_table(z, t_pre, args.arch_seqs, args.arch_prompt,
                                             phases=tuple(args.arch_phases.split(",")))
         result["sizes"][name] = entry
     print(json.dumps(result), flush=True)
