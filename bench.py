@@ -766,8 +766,9 @@ def _gibavik_kernel_table(z, t_pre, n_dec, ctx, phases=("prefill", "decode")):
                                                                                         128, 128)), bytes_=prep_bytes)
         q128 = torch.randn(t, h * 128, device=dev).to(bf)
         g128 = qkv[:, (h + 16) * 128:]
+        vturn = torch.randn(t, 128, device=dev)
         r1, r2 = torch.full((h,), 0.5, device=dev), torch.full((h,), 0.1, device=dev)
-        us_win = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 50.0, h, 8, 128, 128, window=window, vfreq=vfr, gate=g128), reps)
+        us_win = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 50.0, h, 8, 128, 128, window=window, v_turn=vturn, gate=g128), reps)
         us_pen = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 0.0, h, 8, 128, 128, r1=r1, r2=r2), reps)
         us_plain = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 30.0, h, 8, 128, 128), reps)
         kc4, vc4 = kc.view(n_rows, 8, 128), vc.view(n_rows, 8, 128)

@@ -530,15 +530,19 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  *     dim, k_w: kv_heads * dim entries); 0: none.  Then the first rot_dims of every q and k head are turned in pairs by positions[t] *
  *     freq[m], pair m = (m, m + rot_dims / 2) or (2m, 2m + 1) if `interleaved`; with vfreq (vdim / 2 entries) every value head is
  *     turned over all of vdim by positions[t] * vfreq[m] in the same pair layout.  q_out[t], k_cache[slots[t]], v_cache[slots[t]]
- *     take the results; a negative slot stores no key or value.
+ *     take the results; a negative slot stores no key or value.  vcs_out (n_tok, vdim) float32, if given with vfreq, receives every
+ *     token's cos | sin (vdim / 2 each) of positions[t] * vfreq[m]: the table nvx_softcap_attn turns its read-out back with.
  * nvx_softcap_attn:  token t of sequence b attends over the rows at slots kv_indices[kv_start[b] + j], j <= kv_len[b] - q_len[b] +
  *     (t - qo_indptr[b]) (and, with window > 0, only the last `window` of them: itself and the window - 1 before it):
  *     s_j = scale * q . k_j,  s_j <- cap tanh(s_j / cap) (cap > 0),  s_j <- s_j - r1[h] ln(1 + r2[h] (i - j)) (r1, r2 != null; i the
- *     query's position),  out = softmax(s) V; with vfreq the pairs of out are turned by -i * vfreq[m] (the counterpart of
- *     nvx_attn_prep_store's rotated values), with gate out is multiplied by sigmoid(gate[t]) (same layout as out).  Query head h reads
+ *     query's position),  out = softmax(s) V; with vcs ((n_tok, vdim) float32: each query token's cos | sin, as nvx_attn_prep_store
+ *     hands them out) the pairs of out are turned back by those angles (the counterpart of rotated values), with gate out is multiplied by sigmoid(gate[t]) (same layout as out).  Query head h reads
  *     key/value head h / (heads / kv_heads).  q (n_tok, heads * dim), k_cache (slots, kv_heads * dim), v_cache (slots, kv_heads *
  *     vdim), out (n_tok, heads * vdim).  n_split > 1 (for steps of few tokens): a (token, head)'s keys are dealt out over n_split
  *     workgroups whose partial results go to `part` (n_tok * heads * n_split * (vdim + 2) floats) and are merged by a second launch.
+ *     With matrix_cores != 0, a ragged step (qo_indptr given, n_seq sequences), n_split == 1 and sizes for which
+ *     nvx_softcap_attn_tile_fits answers 1, the products run on the matrix cores (64 query tokens of a sequence per workgroup,
+ *     keys in tiles of 32, weights as hi + lo 16-bit halves); scores and the softmax stay float32.
  * nvx_moe_route:  idx[t][k], wts[t][k] = the expert with the k-th largest logit of token t (ties: the lower id) and the sigmoid
  *     of that logit.
  * Expert e:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + shift), result W_down y, with
@@ -553,7 +557,9 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  * nvx_moe_glu:  y[r][j] = the expert's activation of (gu[r][j], gu[r][ff + j]).
  * nvx_moe_gather_rows:  out[t] = sum_k wts[t * top + k] * ys[dst[t * top + k]] (wts == null: ones).
  * nvx_decay_scan:  x[t] holds q at q_off, k at k_off (heads * dim each) and v at v_off (heads * vdim); act 1: silu of all three first.
- *     S <- decay[h] S + k v^T;  out[t] = S^T q.   S (slots, heads, dim, vdim), decay (heads) float32.  dim <= 512.
+ *     S <- decay[h] S + k v^T;  out[t] = S^T q.   S (slots, heads, dim, vdim), decay (heads) float32.  dim <= 512.  chunk > 0 (ragged
+ *     steps): portions are cut into chunks of that many tokens which run side by side, the states at their starts carried through
+ *     ws (n_seq * n_chunk_max * heads * dim * vdim floats; n_chunk_max >= the chunks of the longest portion); chunk 0: one walk.
  * nvx_postnorm_residual:  r = a y[t] (+ b y2[t]);  x[t] += r / rms(r) * w_post (w_post_n = 1: one number, = width: per channel);
  *     h_out[t] = x[t] / rms(x[t]) * w_next (w_next != null) or x[t] itself, in the format `fmt`.  rms(z) = sqrt(mean z^2 + eps).
  * nvx_embed_scale:  x[t] = table[ids[t]] * scale (float32), h[t] the same in the table's format (h may be null).
@@ -594,17 +600,18 @@ int nvx_rope_vnorm_store(const void* x, int64_t x_stride, int fmt, const int64_t
 int nvx_softcap_attn(const void* q, const void* k_cache, const void* v_cache, int fmt, const int32_t* kv_indices,
                      const int64_t* kv_start, const int32_t* kv_len, const int32_t* qo_indptr, const int32_t* tok_seq,
                      float scale, float cap, void* out, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
-                     int n_split, float* part, int64_t window, const float* r1, const float* r2, const double* vfreq,
-                     int v_interleaved, const void* gate, int64_t gate_stride, nvx_stream_t stream);
+                     int n_split, float* part, int64_t window, const float* r1, const float* r2, const float* vcs,
+                     int v_interleaved, const void* gate, int64_t gate_stride, int64_t n_seq, int matrix_cores, nvx_stream_t stream);
+int nvx_softcap_attn_tile_fits(int fmt, int64_t dim, int64_t vdim, int turned_halves);
 int nvx_attn_prep_store(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off,
                         const int64_t* positions, const float* q_w, const float* k_w, int norm_mode, float eps, const double* freq,
                         int rot_dims, int interleaved, const double* vfreq, const int64_t* slots, void* q_out, void* k_cache,
                         void* v_cache, int64_t n_slots, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
-                        nvx_stream_t stream);
+                        float* vcs_out, nvx_stream_t stream);
 int nvx_decay_scan(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off, int act,
                    const float* decay, float* S, int64_t n_slots, const int32_t* qo_indptr, const int64_t* pos0,
                    const int32_t* state_slot, float* out, int64_t n_tok, int64_t n_seq, int64_t heads, int64_t dim, int64_t vdim,
-                   nvx_stream_t stream);
+                   int64_t chunk, int64_t n_chunk_max, float* ws, nvx_stream_t stream);
 int nvx_postnorm_residual(const void* y, int64_t y_stride, const void* y2, int64_t y2_stride, float a, float b, const float* w_post,
                           int64_t w_post_n, int fmt, float* x, const float* w_next, int64_t w_next_n, float eps, void* h_out,
                           int64_t n_tok, int64_t width, nvx_stream_t stream);

@@ -109,11 +109,12 @@ SIGNATURES = {
     "nvx_rope_vnorm_store": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_f32, _c_i32, _c_f32, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64,
                                       _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
     "nvx_softcap_attn": (_c_i32, [_c_vp, _c_vp, _c_vp, _c_i32, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64, _c_i64,
-                                  _c_i64, _c_i64, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_i32, _c_vp, _c_i64, _c_vp]),
+                                  _c_i64, _c_i64, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_i32, _c_vp, _c_i64, _c_i64, _c_i32, _c_vp]),
+    "nvx_softcap_attn_tile_fits": (_c_i32, [_c_i32, _c_i64, _c_i64, _c_i32]),
     "nvx_attn_prep_store": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_vp, _c_i32, _c_f32, _c_vp, _c_i32, _c_i32,
-                                     _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
+                                     _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp]),
     "nvx_decay_scan": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_i64, _c_i64, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp,
-                                _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
+                                _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp]),
     "nvx_postnorm_residual": (_c_i32, [_c_vp, _c_i64, _c_vp, _c_i64, _c_f32, _c_f32, _c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_f32, _c_vp,
                                        _c_i64, _c_i64, _c_vp]),
     "nvx_embed_scale": (_c_i32, [_c_vp, _c_vp, _c_i32, _c_i64, _c_f32, _c_vp, _c_vp, _c_i64, _c_i64, _c_vp]),

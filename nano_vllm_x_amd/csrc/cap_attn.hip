@@ -62,7 +62,8 @@ __global__ __launch_bounds__(256) void rope_vnorm_store_kernel(const A* __restri
 //                heads * dim / kv_heads * dim entries;  0: no norm.
 //   The first rot_dims of every q and k head are then turned in pairs by positions[t] * freq[m]: pair m is (m, m + rot_dims / 2), or
 //   (2m, 2m + 1) if `interleaved`.  With vfreq, every value head is turned the same way over all of vdim by positions[t] * vfreq[m].
-// Angles, cosines and sines are formed in double precision; the norm is float32.
+// Angles, cosines and sines are formed in double precision; the norm is float32.  vcs_out (n_tok, vdim), if given, receives every
+// token's cos | sin of positions[t] * vfreq[m] (vdim / 2 each).
 template <typename A>
 __global__ __launch_bounds__(256) void attn_prep_store_kernel(const A* __restrict__ x, int64_t x_stride, int q_off, int k_off, int v_off,
                                                              const int64_t* __restrict__ positions, const float* __restrict__ q_w,
@@ -70,7 +71,7 @@ __global__ __launch_bounds__(256) void attn_prep_store_kernel(const A* __restric
                                                              const double* __restrict__ freq, int rot_dims, int interleaved,
                                                              const double* __restrict__ vfreq, const int64_t* __restrict__ slots,
                                                              A* __restrict__ q_out, A* __restrict__ k_cache, A* __restrict__ v_cache, int heads,
-                                                             int kv_heads, int dim, int vdim) {
+                                                             int kv_heads, int dim, int vdim, float* __restrict__ vcs_out) {
     extern __shared__ float sm[];
     __shared__ float red[4];
     const int nq = heads * dim, nk = kv_heads * dim, nv = kv_heads * vdim;
@@ -86,11 +87,13 @@ __global__ __launch_bounds__(256) void attn_prep_store_kernel(const A* __restric
         cs[i] = (float)cos(a);
         cs[half + i] = (float)sin(a);
     }
-    if (vfreq && nv)
+    if (vfreq)                          // also handed out (vcs_out[t] = cos | sin): the attention turns its read-out back by the same angles
         for (int i = threadIdx.x; i < vhalf; i += 256) {
             const double a = pos * vfreq[i];
-            vcs[i] = (float)cos(a);
-            vcs[vhalf + i] = (float)sin(a);
+            const float cv = (float)cos(a), sv = (float)sin(a);
+            vcs[i] = cv;
+            vcs[vhalf + i] = sv;
+            if (vcs_out) { vcs_out[t * (int64_t)vdim + i] = cv; vcs_out[t * (int64_t)vdim + vhalf + i] = sv; }
         }
     for (int i = threadIdx.x; i < nq + nk; i += 256) buf[i] = ld_f(row, i < nq ? q_off + i : k_off + (i - nq));
     __syncthreads();
@@ -150,18 +153,17 @@ __global__ __launch_bounds__(256) void attn_prep_store_kernel(const A* __restric
 }
 
 // The end of an attention read-out for one (token, head): `so` holds its vdim values in LDS (every thread of the workgroup has
-// passed a barrier since they were written).  With vfreq the pairs are turned BACK by pos * vfreq[m] (values were cached turned
-// by their own positions, so the weighted sum is a sum of values in the query's frame); with a gate row every element is
-// multiplied by sigmoid(gate).
+// passed a barrier since they were written).  With `turn` (the query token's cos | sin row, vdim / 2 each, as nvx_attn_prep_store
+// hands it out) the pairs are turned BACK by those angles (values were cached turned by their own positions, so the weighted sum
+// is a sum of values in the query's frame); with a gate row every element is multiplied by sigmoid(gate).
 template <typename A>
-__device__ __forceinline__ void attn_readout_end(float* so, int vdim, int64_t pos, const double* __restrict__ vfreq, int interleaved,
+__device__ __forceinline__ void attn_readout_end(float* so, int vdim, const float* __restrict__ turn, int interleaved,
                                                  const A* __restrict__ gate_row, A* __restrict__ out_row, int n_threads) {
-    if (vfreq) {
+    if (turn) {
         const int vhalf = vdim / 2;
         for (int m = threadIdx.x; m < vhalf; m += n_threads) {
             const int i0 = interleaved ? 2 * m : m, i1 = interleaved ? 2 * m + 1 : m + vhalf;
-            const double a = (double)pos * vfreq[m];
-            const float c = (float)cos(a), s = (float)sin(a);
+            const float c = turn[m], s = turn[vhalf + m];
             const float u = so[i0], v = so[i1];
             so[i0] = u * c + v * s;
             so[i1] = v * c - u * s;
@@ -189,7 +191,7 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
                                                           const int32_t* __restrict__ tok_seq, float scale, float cap, A* __restrict__ out,
                                                           int heads, int kv_heads, int dim, int vdim, int vec_v_ok, int n_split,
                                                           float* __restrict__ part, int window, const float* __restrict__ r1,
-                                                          const float* __restrict__ r2, const double* __restrict__ vfreq, int v_inter,
+                                                          const float* __restrict__ r2, const float* __restrict__ vcs, int v_inter,
                                                           const A* __restrict__ gate, int64_t gate_stride) {
     extern __shared__ float sm[];
     float* sq = sm;                   // dim
@@ -309,22 +311,256 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
 #pragma unroll
         for (int w = 0; w < 4; ++w) o += sacc[w * vdim + e] * f[w];
         if (pr) pr[2 + e] = o;
-        else if (vfreq || gate) sacc[e] = o / total;          // (this thread alone reads column e of the four partial sums)
+        else if (vcs || gate) sacc[e] = o / total;            // (this thread alone reads column e of the four partial sums)
         else st_f(out, t * (int64_t)heads * vdim + (int64_t)hd * vdim + e, o / total);
     }
     if (pr && threadIdx.x == 0) { pr[0] = mm; pr[1] = total; }
-    if (!pr && (vfreq || gate)) {
+    if (!pr && (vcs || gate)) {
         __syncthreads();
-        attn_readout_end<A>(sacc, vdim, visible - 1, vfreq, v_inter, gate ? gate + t * gate_stride + (int64_t)hd * vdim : nullptr,
+        attn_readout_end<A>(sacc, vdim, vcs ? vcs + t * (int64_t)vdim : nullptr, v_inter, gate ? gate + t * gate_stride + (int64_t)hd * vdim : nullptr,
                             out + t * (int64_t)heads * vdim + (int64_t)hd * vdim, 256);
+    }
+}
+
+// ---- the same attention on the matrix cores, for steps of many tokens in a 16-bit format -------------------------------------
+// A workgroup takes 64 consecutive query tokens of ONE sequence and one query head; each of its four waves owns 16 of them.  Keys
+// are walked in tiles of 32.  Per tile and wave:
+//   S^T (16 keys x 16 queries), twice = K_tile (16 x dim) . Q^T (dim x 16)      v_mfma_f32_16x16x32, dim / 32 of them each; the A
+//       operand comes straight from the cache rows (lane (key, quarter) takes 16 bytes per step), fetched one tile ahead, the B
+//       operand (the wave's queries) stays in registers;
+//   the result leaves every lane with ONE query (lane & 15) and eight keys (4 * quarter + r of both halves): scale, cap, penalty,
+//       mask, running maximum and sum are float32 per lane, reduced over the quarters by lane exchange;
+//   O^T (vdim x 16 queries) += V_tile^T (vdim x 32 keys) . P^T (32 keys x 16 queries)      v_mfma_f32_16x16x32, vdim / 16 of them, twice:
+//       the weights stay float32 up to here and enter as hi + lo, which keeps 16 bits of their mantissa; P^T is what the lane
+//       holds (its eight keys in the order quarter-of-half-0, quarter-of-half-1), and V^T is read from an LDS tile in that same key
+//       order; the tile is written transposed by the whole workgroup, once for its four waves.
+// At the end a lane holds, for its query, value columns 16 * tile + 4 * quarter + r: both partners of a pair that is turned back
+// (halves: tiles vt and vt + VT / 2; side by side: r and r + 1) are in the lane, so the read-out's end needs no exchange.
+typedef __attribute__((ext_vector_type(8))) __bf16 ca_bf16x8;
+typedef __attribute__((ext_vector_type(8))) _Float16 ca_f16x8;
+template <typename A> __device__ __forceinline__ nvx_f32x4 ca_mfma32(nvx_u32x4 a, nvx_u32x4 b, nvx_f32x4 c) {
+    if constexpr (__is_same(A, __bf16))
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(ca_bf16x8, a), __builtin_bit_cast(ca_bf16x8, b), c, 0, 0, 0);
+    else
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(ca_f16x8, a), __builtin_bit_cast(ca_f16x8, b), c, 0, 0, 0);
+}
+template <typename A> __device__ __forceinline__ uint32_t ca_pack2(float lo, float hi) {
+    typedef float f2 __attribute__((ext_vector_type(2)));
+    typedef A a2 __attribute__((ext_vector_type(2)));
+    const f2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, a2));
+}
+
+constexpr int TILE_Q = 64;       // query tokens per workgroup
+constexpr int TILE_K = 32;       // keys per step
+constexpr int VT_ROW = 40;       // elements per row of the V^T tile in LDS: 32 keys and a pad that spreads the rows over the banks
+
+template <typename A, int DS, int VT>
+__global__ __launch_bounds__(256) void softcap_attn_tile_kernel(const A* __restrict__ q, const A* __restrict__ k_cache, const A* __restrict__ v_cache,
+                                                               const int32_t* __restrict__ kv_indices, const int64_t* __restrict__ kv_start,
+                                                               const int32_t* __restrict__ kv_len, const int32_t* __restrict__ qo_indptr, int n_seq,
+                                                               float scale, float cap, A* __restrict__ out, int heads, int kv_heads, int window,
+                                                               const float* __restrict__ r1, const float* __restrict__ r2,
+                                                               const float* __restrict__ vcs, int v_inter, const A* __restrict__ gate,
+                                                               int64_t gate_stride) {
+    constexpr int dim = DS * 32, vdim = VT * 16;
+    __shared__ A vt_lds[vdim * VT_ROW];
+    __shared__ int where[2];
+    if (threadIdx.x == 0) {          // which sequence and which block of its tokens: sequences take ceil(tokens / 64) workgroups each
+        int rem = blockIdx.x, found = -1;
+        for (int b = 0; b < n_seq; ++b) {
+            const int nb = (qo_indptr[b + 1] - qo_indptr[b] + TILE_Q - 1) / TILE_Q;
+            if (rem < nb) { found = b; break; }
+            rem -= nb;
+        }
+        where[0] = found;
+        where[1] = rem;
+    }
+    __syncthreads();
+    const int b = where[0];
+    if (b < 0) return;               // (the grid is an upper bound)
+    const int hd = blockIdx.y, kvh = hd / (heads / kv_heads);
+    const int q0 = qo_indptr[b], q_n = qo_indptr[b + 1] - q0, qs = where[1] * TILE_Q;
+    const int rows_here = q_n - qs < TILE_Q ? q_n - qs : TILE_Q;
+    const int pos_first = kv_len[b] - q_n + qs;                 // position of the block's first query
+    const int hi = pos_first + rows_here;                       // keys [lo, hi) are seen by some query of the block
+    const int lo = window > 0 && pos_first - window + 1 > 0 ? pos_first - window + 1 : 0;
+    const int32_t* slots = kv_indices + kv_start[b];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+    const int row = wave * 16 + c;
+    const bool row_on = row < rows_here;
+    const int pos = pos_first + row;
+    const int w_hi = pos_first + wave * 16 + 16 < hi ? pos_first + wave * 16 + 16 : hi;      // this wave's queries see [w_lo, w_hi)
+    const int w_lo = window > 0 && pos_first + wave * 16 - window + 1 > 0 ? pos_first + wave * 16 - window + 1 : 0;
+    const bool wave_on = wave * 16 < rows_here;
+    const int64_t k_row = (int64_t)kv_heads * dim, v_row = (int64_t)kv_heads * vdim;
+    nvx_u32x4 qb[DS];
+    {
+        const A* qr = q + ((int64_t)q0 + qs + (row_on ? row : rows_here - 1)) * heads * dim + (int64_t)hd * dim + 8 * g;
+#pragma unroll
+        for (int s = 0; s < DS; ++s) qb[s] = *reinterpret_cast<const nvx_u32x4*>(qr + 32 * s);
+    }
+    const float pen_a = r1 ? r1[hd] : 0.f, pen_b = r1 ? r2[hd] : 0.f;
+    nvx_f32x4 acc[VT];
+#pragma unroll
+    for (int t = 0; t < VT; ++t) acc[t] = nvx_f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    // Rows hang on slot ids, which hang on the slot list: two memory round trips in a row.  The ids are read two tiles ahead and the
+    // rows one tile ahead (keys into the registers the products read, values into registers that the next step writes to LDS),
+    // so that neither wait stands in front of a tile's products.
+    constexpr int VCH = TILE_K * (vdim / 8);                         // 16-byte pieces of a tile of values
+    constexpr int VPT = (VCH + 255) / 256;                           // ... per thread
+    typedef A vec8 __attribute__((ext_vector_type(8)));
+    nvx_u32x4 kf[2][DS];
+    vec8 vf[VPT];
+    int k_slot[2], v_slot[VPT];
+    auto fetch_slots = [&](int j0) {                                 // (a key past the end reads a real row and is masked)
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) { const int j = j0 + hh * 16 + c; k_slot[hh] = slots[j < hi ? j : hi - 1]; }
+#pragma unroll
+        for (int u = 0; u < VPT; ++u) { const int j = j0 + ((threadIdx.x + 256 * u) & (TILE_K - 1)); v_slot[u] = slots[j < hi ? j : hi - 1]; }
+    };
+    auto fetch_rows = [&]() {
+        if (wave_on) {
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                const A* kr = k_cache + (int64_t)k_slot[hh] * k_row + (int64_t)kvh * dim + 8 * g;
+#pragma unroll
+                for (int s = 0; s < DS; ++s) kf[hh][s] = *reinterpret_cast<const nvx_u32x4*>(kr + 32 * s);
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < VPT; ++u) {
+            const int i = threadIdx.x + 256 * u;
+            if (i < VCH) vf[u] = *reinterpret_cast<const vec8*>(v_cache + (int64_t)v_slot[u] * v_row + (int64_t)kvh * vdim + (i / TILE_K) * 8);
+        }
+    };
+    const int j_begin = lo & ~(TILE_K - 1);
+    fetch_slots(j_begin);
+    fetch_rows();
+    if (j_begin + TILE_K < hi) fetch_slots(j_begin + TILE_K);
+    for (int j0 = j_begin; j0 < hi; j0 += TILE_K) {
+        __syncthreads();                                             // the tile before has been read by all waves
+#pragma unroll
+        for (int u = 0; u < VPT; ++u) {
+            const int i = threadIdx.x + 256 * u;
+            if (i < VCH) {
+                const int kk = i & (TILE_K - 1), ch = i / TILE_K;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) vt_lds[(ch * 8 + e) * VT_ROW + kk] = vf[u][e];
+            }
+        }
+        nvx_u32x4 kc[2][DS];
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+            for (int s = 0; s < DS; ++s) kc[hh][s] = kf[hh][s];
+        if (j0 + TILE_K < hi) fetch_rows();                          // (with the ids read one step ago)
+        if (j0 + 2 * TILE_K < hi) fetch_slots(j0 + 2 * TILE_K);
+        __syncthreads();
+        if (!wave_on) continue;
+        if (j0 >= w_hi || j0 + TILE_K <= w_lo) continue;            // none of this wave's queries sees the tile
+        float sv[8], mx = -INFINITY;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            nvx_f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int s = 0; s < DS; ++s) sacc = ca_mfma32<A>(kc[hh][s], qb[s], sacc);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int j = j0 + hh * 16 + 4 * g + r;
+                float sc = -INFINITY;
+                if (row_on && j <= pos && (window <= 0 || j > pos - window)) {
+                    sc = sacc[r] * scale;
+                    if (cap > 0.f) sc = cap * (1.0f - 2.0f / (__expf(2.0f * sc / cap) + 1.0f));      // tanh by the hardware exponential
+                    if (r1) sc -= pen_a * __logf(1.0f + pen_b * (float)(pos - j));
+                }
+                sv[hh * 4 + r] = sc;
+                mx = fmaxf(mx, sc);
+            }
+        }
+        mx = fmaxf(mx, xor16(mx));
+        mx = fmaxf(mx, xor32(mx));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = m_new == -INFINITY ? 1.0f : __expf(m_run - m_new);    // (nothing seen yet: nothing to rescale)
+        m_run = m_new;
+        l_run *= alpha;
+        float p[8], ph[8];
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            p[e] = sv[e] == -INFINITY ? 0.f : __expf(sv[e] - m_new);
+            l_run += p[e];
+            ph[e] = (float)(A)p[e];
+        }
+        const nvx_u32x4 p_hi = {ca_pack2<A>(ph[0], ph[1]), ca_pack2<A>(ph[2], ph[3]), ca_pack2<A>(ph[4], ph[5]), ca_pack2<A>(ph[6], ph[7])};
+        const nvx_u32x4 p_lo = {ca_pack2<A>(p[0] - ph[0], p[1] - ph[1]), ca_pack2<A>(p[2] - ph[2], p[3] - ph[3]),
+                                ca_pack2<A>(p[4] - ph[4], p[5] - ph[5]), ca_pack2<A>(p[6] - ph[6], p[7] - ph[7])};
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int t = 0; t < VT; ++t) acc[t] *= alpha;
+        }
+#pragma unroll
+        for (int t = 0; t < VT; ++t) {
+            // row (value column) 16 t + c of V^T, keys 4 g .. 4 g + 3 of both halves: the order of the lane's weights
+            const A* vr = vt_lds + (t * 16 + c) * VT_ROW + 4 * g;
+            const uint2 a0 = *reinterpret_cast<const uint2*>(vr), a1 = *reinterpret_cast<const uint2*>(vr + 16);
+            const nvx_u32x4 vfrag = {a0.x, a0.y, a1.x, a1.y};
+            acc[t] = ca_mfma32<A>(vfrag, p_hi, acc[t]);
+            acc[t] = ca_mfma32<A>(vfrag, p_lo, acc[t]);
+        }
+    }
+    if (!wave_on) return;
+    l_run += xor16(l_run);
+    l_run += xor32(l_run);
+    if (!row_on) return;
+    const float inv = 1.0f / l_run;
+#pragma unroll
+    for (int t = 0; t < VT; ++t) acc[t] *= inv;
+    const int64_t tok = (int64_t)q0 + qs + row;
+    if (vcs) {
+        const float* cs = vcs + tok * vdim, *sn = cs + vdim / 2;
+        if (v_inter) {
+#pragma unroll
+            for (int t = 0; t < VT; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; r += 2) {
+                    const int m = (t * 16 + 4 * g + r) >> 1;
+                    const float u = acc[t][r], v = acc[t][r + 1];
+                    acc[t][r] = u * cs[m] + v * sn[m];
+                    acc[t][r + 1] = v * cs[m] - u * sn[m];
+                }
+        } else {
+#pragma unroll
+            for (int t = 0; t < VT / 2; ++t) {
+                const nvx_f32x4 c4 = *reinterpret_cast<const nvx_f32x4*>(cs + t * 16 + 4 * g), s4 = *reinterpret_cast<const nvx_f32x4*>(sn + t * 16 + 4 * g);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float u = acc[t][r], v = acc[t + VT / 2][r];
+                    acc[t][r] = u * c4[r] + v * s4[r];
+                    acc[t + VT / 2][r] = v * c4[r] - u * s4[r];
+                }
+            }
+        }
+    }
+    A* orow = out + tok * heads * vdim + (int64_t)hd * vdim + 4 * g;
+    const A* grow = gate ? gate + tok * gate_stride + (int64_t)hd * vdim + 4 * g : nullptr;
+#pragma unroll
+    for (int t = 0; t < VT; ++t) {
+        float o[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+        if (grow) {
+            typedef A vec4 __attribute__((ext_vector_type(4)));
+            const vec4 gv = *reinterpret_cast<const vec4*>(grow + t * 16);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[r] *= sigmoid_f((float)gv[r]);
+        }
+        *reinterpret_cast<uint2*>(orow + t * 16) = make_uint2(ca_pack2<A>(o[0], o[1]), ca_pack2<A>(o[2], o[3]));
     }
 }
 
 // out = the n_split partial results of a (token, head) merged: each is (maximum, sum, unnormalised values); one wave each.
 template <typename A>
 __global__ __launch_bounds__(64) void softcap_merge_kernel(const float* __restrict__ part, int n_split, A* __restrict__ out, int vdim,
-                                                          int heads, const int32_t* __restrict__ kv_len, const int32_t* __restrict__ qo_indptr,
-                                                          const int32_t* __restrict__ tok_seq, const double* __restrict__ vfreq, int v_inter,
+                                                          int heads, const float* __restrict__ vcs, int v_inter,
                                                           const A* __restrict__ gate, int64_t gate_stride) {
     __shared__ float so[512];
     const int64_t row = blockIdx.x;
@@ -342,23 +578,31 @@ __global__ __launch_bounds__(64) void softcap_merge_kernel(const float* __restri
             const float m = pr[s * (vdim + 2)];
             if (m != -INFINITY) o += pr[s * (vdim + 2) + 2 + e] * expf(m - mm);
         }
-        if (vfreq || gate) so[e] = o / total;
+        if (vcs || gate) so[e] = o / total;
         else st_f(out, row * vdim + e, o / total);
     }
-    if (vfreq || gate) {
+    if (vcs || gate) {
         const int64_t t = row / heads;
-        const int b = tok_seq ? tok_seq[t] : (int)t;
-        const int64_t q0 = qo_indptr ? qo_indptr[b] : b;
-        const int64_t q_n = qo_indptr ? qo_indptr[b + 1] - q0 : 1;
-        const int64_t pos = kv_len[b] - (q_n - 1 - (t - q0)) - 1;
         __syncthreads();
-        attn_readout_end<A>(so, vdim, pos, vfreq, v_inter, gate ? gate + t * gate_stride + (row % heads) * vdim : nullptr, out + row * vdim, 64);
+        attn_readout_end<A>(so, vdim, vcs ? vcs + t * (int64_t)vdim : nullptr, v_inter, gate ? gate + t * gate_stride + (row % heads) * vdim : nullptr,
+                            out + row * vdim, 64);
     }
 }
 
 }  // namespace NVX_NS
 
 using namespace NVX_NS;
+
+// the tile kernel is built for 16-bit formats only; float stands in so that the format dispatch compiles (never launched)
+template <typename T> struct tile_fmt { typedef T type; };
+template <> struct tile_fmt<float> { typedef __bf16 type; };
+
+// Whether nvx_softcap_attn has a matrix-core form for these sizes: 16-bit formats, key and value sizes of 64, 96 or 128; a read-out
+// that is turned back in the halves layout needs both halves in whole column tiles.
+extern "C" int nvx_softcap_attn_tile_fits(int fmt, int64_t dim, int64_t vdim, int turned_halves) {
+    const bool sizes = (dim == 64 || dim == 96 || dim == 128) && (vdim == 64 || vdim == 96 || vdim == 128);
+    return (fmt == 0 || fmt == 1) && sizes && (!turned_halves || (vdim / 16) % 2 == 0);
+}
 
 extern "C" int nvx_rope_vnorm_store(const void* x, int64_t x_stride, int fmt, const int64_t* positions, const double* freq, float mag,
                                     int rot_dims, float eps, const int64_t* slots, void* q_out, void* k_cache, void* v_cache,
@@ -382,7 +626,7 @@ extern "C" int nvx_attn_prep_store(const void* x, int64_t x_stride, int fmt, int
                                    const int64_t* positions, const float* q_w, const float* k_w, int norm_mode, float eps, const double* freq,
                                    int rot_dims, int interleaved, const double* vfreq, const int64_t* slots, void* q_out, void* k_cache,
                                    void* v_cache, int64_t n_slots, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
-                                   nvx_stream_t stream) {
+                                   float* vcs_out, nvx_stream_t stream) {
     NVX_REQUIRE(fmt >= 0 && fmt <= 2 && norm_mode >= 0 && norm_mode <= 2, NVX_EINVAL, "nvx_attn_prep_store: fmt must be 0..2, norm_mode 0..2");
     NVX_REQUIRE(n_tok >= 0 && heads > 0 && kv_heads >= 0 && dim > 0 && vdim > 0 && n_slots >= 0, NVX_EINVAL, "nvx_attn_prep_store: bad sizes");
     const int64_t nq = heads * dim, nk = kv_heads * dim, nv = kv_heads * vdim;
@@ -399,15 +643,16 @@ extern "C" int nvx_attn_prep_store(const void* x, int64_t x_stride, int fmt, int
     NVX_FMT_CALL(fmt, hipLaunchKernelGGL(attn_prep_store_kernel<A_>, dim3((unsigned)n_tok), dim3(256), lds, (hipStream_t)stream, (const A_*)x, x_stride,
                                          (int)q_off, (int)k_off, (int)v_off, positions, q_w, k_w, norm_mode, eps, freq, rot_dims, interleaved, vfreq,
                                          kv_heads ? slots : nullptr, (A_*)q_out, (A_*)k_cache, (A_*)v_cache, (int)heads, (int)kv_heads, (int)dim,
-                                         (int)vdim));
+                                         (int)vdim, vcs_out));
     return nvx_check_launch("nvx_attn_prep_store");
 }
 
 extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* v_cache, int fmt, const int32_t* kv_indices,
                                 const int64_t* kv_start, const int32_t* kv_len, const int32_t* qo_indptr, const int32_t* tok_seq,
                                 float scale, float cap, void* out, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
-                                int n_split, float* part, int64_t window, const float* r1, const float* r2, const double* vfreq,
-                                int v_interleaved, const void* gate, int64_t gate_stride, nvx_stream_t stream) {
+                                int n_split, float* part, int64_t window, const float* r1, const float* r2, const float* vcs,
+                                int v_interleaved, const void* gate, int64_t gate_stride, int64_t n_seq, int matrix_cores,
+                                nvx_stream_t stream) {
     NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_softcap_attn: fmt must be 0, 1 or 2");
     NVX_REQUIRE(n_tok >= 0 && n_tok <= 65535 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && dim <= 4096 && vdim > 0 && vdim <= 512,
                 NVX_EINVAL, "nvx_softcap_attn: bad sizes (at most 65535 tokens a step, key size <= 4096, value size <= 512)");
@@ -416,8 +661,32 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
     NVX_REQUIRE((tok_seq != nullptr) == (qo_indptr != nullptr), NVX_EINVAL, "nvx_softcap_attn: tok_seq and qo_indptr go together");
     NVX_REQUIRE((r1 != nullptr) == (r2 != nullptr), NVX_EINVAL, "nvx_softcap_attn: the distance penalty takes both of its numbers per head");
     NVX_REQUIRE(window >= 0 && window < (1ll << 31), NVX_EINVAL, "nvx_softcap_attn: bad window");
-    NVX_REQUIRE(!vfreq || vdim % 2 == 0, NVX_EINVAL, "nvx_softcap_attn: a read-out that is turned back has an even size");
+    NVX_REQUIRE(!vcs || (vdim % 2 == 0 && nvx_aligned16(vcs)), NVX_EINVAL, "nvx_softcap_attn: a read-out that is turned back has an even size");
     NVX_REQUIRE(!gate || gate_stride >= heads * vdim, NVX_EINVAL, "nvx_softcap_attn: row stride of the gate");
+    // steps of many tokens in a 16-bit format, sizes the tile kernel is built for, 8-byte rows of the gate: the matrix cores
+    if (matrix_cores && nvx_softcap_attn_tile_fits(fmt, dim, vdim, vcs != nullptr && !v_interleaved) && qo_indptr && n_split == 1 && n_seq > 0 &&
+        nvx_aligned16(q) && nvx_aligned16(k_cache) && nvx_aligned16(v_cache) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0 &&
+        (!gate || ((reinterpret_cast<uintptr_t>(gate) & 7u) == 0 && gate_stride % 4 == 0))) {
+        const dim3 tgrid((unsigned)((n_tok + TILE_Q - 1) / TILE_Q + n_seq), (unsigned)heads);
+#define NVX_TILE_ATTN(DS, VT)                                                                                                            \
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL((softcap_attn_tile_kernel<typename tile_fmt<A_>::type, DS, VT>), tgrid, dim3(256), 0, (hipStream_t)stream, \
+                                         (const typename tile_fmt<A_>::type*)q, (const typename tile_fmt<A_>::type*)k_cache,            \
+                                         (const typename tile_fmt<A_>::type*)v_cache, kv_indices, kv_start, kv_len, qo_indptr, (int)n_seq, scale, \
+                                         cap, (typename tile_fmt<A_>::type*)out, (int)heads, (int)kv_heads, (int)window, r1, r2, vcs,    \
+                                         v_interleaved, (const typename tile_fmt<A_>::type*)gate, gate_stride))
+#define NVX_TILE_ATTN_V(DS)                                                       \
+    do {                                                                          \
+        if (vdim == 64) NVX_TILE_ATTN(DS, 4);                                     \
+        else if (vdim == 96) NVX_TILE_ATTN(DS, 6);                                \
+        else NVX_TILE_ATTN(DS, 8);                                                \
+    } while (0)
+        if (dim == 64) NVX_TILE_ATTN_V(2);
+        else if (dim == 96) NVX_TILE_ATTN_V(3);
+        else NVX_TILE_ATTN_V(4);
+#undef NVX_TILE_ATTN_V
+#undef NVX_TILE_ATTN
+        return nvx_check_launch("nvx_softcap_attn");
+    }
     const size_t lds = (size_t)(dim + 4 * vdim + 8) * sizeof(float);
     NVX_REQUIRE(n_split >= 1 && n_split <= 64 && (n_split == 1 || part), NVX_EINVAL, "nvx_softcap_attn: a key split needs its workspace");
     const dim3 grid((unsigned)heads, (unsigned)n_tok, (unsigned)n_split);
@@ -425,7 +694,7 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
     NVX_FMT_CALL(fmt, hipLaunchKernelGGL((softcap_attn_kernel<A_, EPL, VEC && sizeof(A_) == 2>), grid, dim3(256), lds, (hipStream_t)stream,     \
                                          (const A_*)q, (const A_*)k_cache, (const A_*)v_cache, kv_indices, kv_start, kv_len, qo_indptr,      \
                                          tok_seq, scale, cap, (A_*)out, (int)heads, (int)kv_heads, (int)dim, (int)vdim,       \
-                                         (int)nvx_aligned16(v_cache), n_split, part, (int)window, r1, r2, vfreq, v_interleaved, \
+                                         (int)nvx_aligned16(v_cache), n_split, part, (int)window, r1, r2, vcs, v_interleaved,   \
                                          (const A_*)gate, gate_stride))
 #define NVX_CAP_ATTN(EPL) do { if (vec) NVX_CAP_ATTN_V(EPL, true); else NVX_CAP_ATTN_V(EPL, false); } while (0)
     const bool vec = fmt != 2 && dim % 8 == 0 && nvx_aligned16(k_cache);
@@ -436,8 +705,8 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
 #undef NVX_CAP_ATTN_V
     if (n_split > 1)
         NVX_FMT_CALL(fmt, hipLaunchKernelGGL(softcap_merge_kernel<A_>, dim3((unsigned)(n_tok * heads)), dim3(64), 0, (hipStream_t)stream,
-                                             (const float*)part, n_split, (A_*)out, (int)vdim, (int)heads, kv_len, qo_indptr, tok_seq, vfreq,
-                                             v_interleaved, (const A_*)gate, gate_stride));
+                                             (const float*)part, n_split, (A_*)out, (int)vdim, (int)heads, vcs, v_interleaved, (const A_*)gate,
+                                             gate_stride));
 #undef NVX_CAP_ATTN
     return nvx_check_launch("nvx_softcap_attn");
 }

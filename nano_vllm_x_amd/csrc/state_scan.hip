@@ -367,25 +367,38 @@ __global__ __launch_bounds__(256) void rwkv_scan_kernel(const A* __restrict__ rx
 // Linear attention with a constant decay per head.  x[t] holds q at q_off, k at k_off (heads * dim each) and v at v_off (heads *
 // vdim), pre-activations if act == 1 (silu is applied to all three as they are staged), values as they are if act == 0.
 //   S <- decay[h] S + k v^T;  o = S^T q  (the read sees the token's own write).          S: (slots, heads, dim, vdim).
+// Long portions are cut into chunks of `chunk` tokens that run side by side (blockIdx.z = sequence * n_chunk_max + chunk), in three
+// launches: phase 1 builds every chunk's own contribution from a zero state into ws (no read-out), the carry kernel turns ws into
+// the state at every chunk's start (and writes the sequence's final state), phase 3 walks every chunk from there with the read-out.
+// Because the decay is a constant, the carry over a chunk of n tokens is decay^n S + (the chunk's own contribution).  phase 0: one
+// workgroup walks the whole portion (single tokens, short portions).
 __device__ __forceinline__ float scan_act(float z, int act) { return act == 1 ? z * sigmoid_f(z) : z; }
 template <typename A>
 __global__ __launch_bounds__(256) void decay_scan_kernel(const A* __restrict__ x, int64_t x_stride, int q_off, int k_off, int v_off, int act,
                                                         const float* __restrict__ decay, float* __restrict__ S,
                                                         const int32_t* __restrict__ qo_indptr, const int64_t* __restrict__ pos0,
                                                         const int32_t* __restrict__ state_slot, float* __restrict__ out, int heads, int dim,
-                                                        int vdim, int p_lanes) {
+                                                        int vdim, int p_lanes, int phase, int chunk, int n_chunk_max, float* __restrict__ ws) {
     extern __shared__ float sm[];
     const int cb = blockDim.x / p_lanes, rs = p_lanes * KS;
     float* sq = sm;
     float* sk = sq + TB * rs;
     float* sv = sk + TB * rs;
     const int hd = blockIdx.y;
-    const SeqSpan sp = seq_span(blockIdx.z, qo_indptr, pos0, state_slot);
+    const int seq = phase ? blockIdx.z / n_chunk_max : blockIdx.z, ck = phase ? blockIdx.z % n_chunk_max : 0;
+    SeqSpan sp = seq_span(seq, qo_indptr, pos0, state_slot);
     if (sp.slot < 0 || sp.n <= 0) return;
+    if (phase) {                                     // this workgroup's chunk of the portion
+        const int64_t first = (int64_t)ck * chunk;
+        if (first >= sp.n) return;
+        sp.q0 += first;
+        sp.n = sp.n - first < chunk ? sp.n - first : chunk;
+    }
     const ScanThread th = scan_thread(p_lanes, vdim);
-    float* Sp = S + ((int64_t)sp.slot * heads + hd) * dim * vdim;
+    // where the state comes from and goes to: the pool (phase 0), nothing and ws (1), ws and nothing (3)
+    float* Sp = phase ? ws + ((int64_t)blockIdx.z * heads + hd) * dim * vdim : S + ((int64_t)sp.slot * heads + hd) * dim * vdim;
     float s[KR];
-    const bool cont = sp.pos0 > 0;
+    const bool cont = phase == 3 || (phase == 0 && sp.pos0 > 0);
 #pragma unroll
     for (int r = 0; r < KR; ++r) {
         const int row = th.r0 + r;
@@ -418,15 +431,43 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(const A* __restrict__ x
                 s[r] = g * s[r] + kk[r] * v;
                 o += s[r] * qq[r];
             }
+            if (phase == 1) continue;                // (only the state is wanted)
             o = lanes_sum(o, p_lanes);
             if (th.p == 0 && th.active) out[(sp.q0 + t0 + tt) * (int64_t)heads * vdim + (int64_t)hd * vdim + th.e] = o;
         }
     }
+    if (phase == 3) return;
 #pragma unroll
     for (int r = 0; r < KR; ++r) {
         const int row = th.r0 + r;
         if (row < dim && th.active) Sp[(int64_t)row * vdim + th.e] = s[r];
     }
+}
+
+// Between the two chunked phases: ws[sequence][chunk] holds every chunk's own contribution and is replaced by the state at the chunk's
+// start; the state after the last chunk goes to the pool.  One thread per element of a sequence's state.
+__global__ __launch_bounds__(256) void decay_chunk_carry_kernel(const float* __restrict__ decay, float* __restrict__ S, float* __restrict__ ws,
+                                                               const int32_t* __restrict__ qo_indptr, const int64_t* __restrict__ pos0,
+                                                               const int32_t* __restrict__ state_slot, int heads, int dim, int vdim, int chunk,
+                                                               int n_chunk_max) {
+    const SeqSpan sp = seq_span(blockIdx.y, qo_indptr, pos0, state_slot);
+    if (sp.slot < 0 || sp.n <= 0) return;
+    const int64_t per = (int64_t)heads * dim * vdim;
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= per) return;
+    const float g = decay[i / ((int64_t)dim * vdim)];
+    float* Sp = S + (int64_t)sp.slot * per + i;
+    float run = sp.pos0 > 0 ? *Sp : 0.f;
+    for (int ck = 0; (int64_t)ck * chunk < sp.n; ++ck) {
+        const int64_t n = sp.n - (int64_t)ck * chunk < chunk ? sp.n - (int64_t)ck * chunk : chunk;
+        float* w = ws + ((int64_t)blockIdx.y * n_chunk_max + ck) * per + i;
+        const float own = *w;
+        *w = run;
+        float gn = 1.f;
+        for (int64_t k = 0; k < n; ++k) gn *= g;     // the same products, in the same order, as n steps of the recurrence
+        run = gn * run + own;
+    }
+    *Sp = run;
 }
 
 // launch geometry of the three recurrences: lanes per column (a power of two), threads per workgroup, value columns per
@@ -561,7 +602,7 @@ extern "C" int nvx_rwkv_scan(const void* r, const void* k, const void* v, int64_
 extern "C" int nvx_decay_scan(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off, int act,
                               const float* decay, float* S, int64_t n_slots, const int32_t* qo_indptr, const int64_t* pos0,
                               const int32_t* state_slot, float* out, int64_t n_tok, int64_t n_seq, int64_t heads, int64_t dim, int64_t vdim,
-                              nvx_stream_t stream) {
+                              int64_t chunk, int64_t n_chunk_max, float* ws, nvx_stream_t stream) {
     NVX_LAYOUT_OK("nvx_decay_scan");
     ScanLaunch g;
     NVX_REQUIRE(heads > 0 && heads <= 65535 && dim > 0 && vdim > 0 && vdim < (1 << 24) && n_slots >= 0 && (act == 0 || act == 1), NVX_EINVAL,
@@ -571,9 +612,22 @@ extern "C" int nvx_decay_scan(const void* x, int64_t x_stride, int fmt, int64_t 
     NVX_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && x_stride >= q_off + heads * dim && x_stride >= k_off + heads * dim &&
                     x_stride >= v_off + heads * vdim, NVX_EINVAL, "nvx_decay_scan: q, k or v lies outside a row");
     const size_t lds = (size_t)(2 * TB * g.p_lanes * KS + TB * g.cb) * sizeof(float);
-    const dim3 grid((unsigned)((vdim + g.cb - 1) / g.cb), (unsigned)heads, (unsigned)n_seq);
-    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(decay_scan_kernel<A_>, grid, dim3(g.threads), lds, (hipStream_t)stream, (const A_*)x, x_stride, (int)q_off,
-                                         (int)k_off, (int)v_off, act, decay, S, qo_indptr, pos0, state_slot, out, (int)heads, (int)dim, (int)vdim,
-                                         g.p_lanes));
+    NVX_REQUIRE(chunk == 0 || (chunk > 0 && chunk < (1 << 30) && n_chunk_max > 0 && n_seq * n_chunk_max <= 65535 && ws && qo_indptr), NVX_EINVAL,
+                "nvx_decay_scan: chunks need a ragged step, their workspace, and at most 65535 of them");
+    const dim3 grid((unsigned)((vdim + g.cb - 1) / g.cb), (unsigned)heads, (unsigned)(chunk ? n_seq * n_chunk_max : n_seq));
+#define NVX_DECAY_SCAN(PHASE)                                                                                                                      \
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(decay_scan_kernel<A_>, grid, dim3(g.threads), lds, (hipStream_t)stream, (const A_*)x, x_stride, (int)q_off, \
+                                         (int)k_off, (int)v_off, act, decay, S, qo_indptr, pos0, state_slot, out, (int)heads, (int)dim, (int)vdim, \
+                                         g.p_lanes, PHASE, (int)chunk, (int)n_chunk_max, ws))
+    if (!chunk) {
+        NVX_DECAY_SCAN(0);
+    } else {
+        NVX_DECAY_SCAN(1);
+        hipLaunchKernelGGL(decay_chunk_carry_kernel, dim3((unsigned)((heads * dim * vdim + 255) / 256), (unsigned)n_seq), dim3(256), 0,
+                           (hipStream_t)stream, decay, S, ws, qo_indptr, pos0, state_slot, (int)heads, (int)dim, (int)vdim, (int)chunk,
+                           (int)n_chunk_max);
+        NVX_DECAY_SCAN(3);
+    }
+#undef NVX_DECAY_SCAN
     return nvx_check_launch("nvx_decay_scan");
 }

@@ -114,11 +114,11 @@ class NormedAttention(nn.Module):
         v0 = k0 + self.k_cols
         g0 = v0 + self.v_cols
         own = not self.borrows
-        q = ops.attn_prep_store(x, (col0, k0, v0), positions, getattr(self, "q_norm", None), getattr(self, "k_norm", None), self.qk_norm, self.eps,
-                                self.freq, self.rot_dims, self.interleaved, self.vfreq if own else None, md.out_slots if own else None,
+        q, v_turn = ops.attn_prep_store(x, (col0, k0, v0), positions, getattr(self, "q_norm", None), getattr(self, "k_norm", None), self.qk_norm, self.eps,
+                                self.freq, self.rot_dims, self.interleaved, self.vfreq, md.out_slots if own else None,
                                 k_cache if own else None, v_cache if own else None, self.heads, self.kv_heads if own else 0, self.dim, self.vdim)
         o = ops.softcap_attn(q, k_cache, v_cache, md.kv_indices, md.kv_start, md.kv_len, md.layout, self.scale, self.softcap, self.heads,
-                             self.kv_heads, self.dim, self.vdim, window=self.window, r1=self.r1, r2=self.r2, vfreq=self.vfreq,
+                             self.kv_heads, self.dim, self.vdim, window=self.window, r1=self.r1, r2=self.r2, v_turn=v_turn,
                              v_interleaved=self.interleaved, gate=x[:, g0:g0 + self.g_cols] if self.out_gate else None)
         return self.o_proj(o)
 

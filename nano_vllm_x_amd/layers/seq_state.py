@@ -75,7 +75,7 @@ class SeqStateBackend:
             qo = np.zeros(n + 1, dtype=np.int32)
             np.cumsum(q_lens, out=qo[1:])
             tok_seq = np.repeat(np.arange(n, dtype=np.int32), q_lens)
-            layout = ops.StepLayout(t, n, self._up(pos0), self._up(slot), self._up(qo), self._up(tok_seq))
+            layout = ops.StepLayout(t, n, self._up(pos0), self._up(slot), self._up(qo), self._up(tok_seq), max_q=int(q_lens.max()))
         kv_indptr = np.zeros(n + 1, dtype=np.int32)
         np.cumsum(kv_lens, out=kv_indptr[1:])
         return SeqStateMetadata(forward_mode=batch.forward_mode, cache=self.cache, layout=layout, kv_indices=self._up(flat),

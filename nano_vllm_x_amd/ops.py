@@ -690,7 +690,7 @@ class StepLayout:
     (both None: one token per sequence, a decode step), `pos0` (int64, B) the position of each sequence's first token of
     the step, `state_slot` (int32, B) its slot in the state tensors (negative: a padding row)."""
 
-    def __init__(self, n_tok: int, n_seq: int, pos0, state_slot, qo_indptr=None, tok_seq=None):
+    def __init__(self, n_tok: int, n_seq: int, pos0, state_slot, qo_indptr=None, tok_seq=None, max_q=None):
         _dev(pos0, state_slot, qo_indptr, tok_seq)
         _need(pos0.dtype == torch.int64 and pos0.is_contiguous() and pos0.numel() >= n_seq, "StepLayout: pos0 must be int64 (B)")
         _need(state_slot.dtype == torch.int32 and state_slot.is_contiguous() and state_slot.numel() >= n_seq,
@@ -703,6 +703,8 @@ class StepLayout:
             _need(tok_seq.dtype == torch.int32 and tok_seq.is_contiguous() and tok_seq.numel() == n_tok, "StepLayout: tok_seq")
         self.n_tok, self.n_seq = n_tok, n_seq
         self.pos0, self.state_slot, self.qo_indptr, self.tok_seq = pos0, state_slot, qo_indptr, tok_seq
+        # tokens of the step's longest portion, where the host knows it (it sizes launches that cut portions into chunks); else n_tok bounds it
+        self.max_q = int(max_q) if max_q else n_tok
 
 
 def boundary_canon_fits(width: int) -> bool:
@@ -1058,22 +1060,24 @@ SOFTCAP_SPLITS = 4
 
 
 def softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, layout: StepLayout, scale: float, cap: float, heads: int,
-                 kv_heads: int, dim: int, vdim: int, n_split: Optional[int] = None, window: int = 0, r1=None, r2=None, vfreq=None,
-                 v_interleaved: bool = False, gate=None):
+                 kv_heads: int, dim: int, vdim: int, n_split: Optional[int] = None, window: int = 0, r1=None, r2=None, v_turn=None,
+                 v_interleaved: bool = False, gate=None, matrix_cores: bool = True):
     """Causal attention of q (T, heads * dim) over cached rows: sequence b's tokens are at slots kv_indices[kv_start[b] :
     kv_start[b] + kv_len[b]]; scores scale * q . k pass cap * tanh(. / cap) (cap <= 0: not) before the softmax.
     `window` > 0: a token sees itself and the window - 1 tokens before it.  `r1`, `r2` (heads, float32): r1 ln(1 + r2 (i - j)) is
-    taken off the score of key j for the query at position i.  `vfreq` (vdim / 2, float64): the read-out's pairs ((m, m + vdim / 2),
-    or (2m, 2m + 1) if `v_interleaved`) are turned by -i * vfreq[m], undoing the turn attn_prep_store gave the values.  `gate`
-    (T, heads * vdim): the read-out times sigmoid(gate).  Returns (T, heads * vdim) in q's format."""
-    _dev(q, k_cache, v_cache, kv_indices, kv_start, kv_len, r1, r2, vfreq, gate)
+    taken off the score of key j for the query at position i.  `v_turn` (T, vdim) float32, every query token's cos | sin as
+    attn_prep_store returns them: the read-out's pairs ((m, m + vdim / 2), or (2m, 2m + 1) if `v_interleaved`) are turned back by
+    those angles, undoing the turn attn_prep_store gave the values.  `gate`
+    (T, heads * vdim): the read-out times sigmoid(gate).  Steps of many tokens in a 16-bit format, with key and value sizes of 64,
+    96 or 128, run on the matrix cores unless `matrix_cores` is False.  Returns (T, heads * vdim) in q's format."""
+    _dev(q, k_cache, v_cache, kv_indices, kv_start, kv_len, r1, r2, v_turn, gate)
     _need((r1 is None) == (r2 is None), "softcap_attn: r1 and r2 go together")
     for a in (r1, r2):
         if a is not None:
             _f32c(a, "softcap_attn: r1, r2")
             _need(a.numel() == heads, "softcap_attn: r1 and r2 have one number per head")
-    _need(vfreq is None or (vfreq.dtype == torch.float64 and vfreq.is_contiguous() and vfreq.numel() == vdim // 2 and vdim % 2 == 0),
-          "softcap_attn: vfreq must be float64 (vdim / 2)")
+    _need(v_turn is None or (v_turn.dtype == F32 and v_turn.is_contiguous() and v_turn.shape == (q.shape[0], vdim) and vdim % 2 == 0),
+          "softcap_attn: v_turn must be float32 (T, vdim)")
     _need(gate is None or (gate.shape == (q.shape[0], heads * vdim) and gate.stride(1) == 1 and gate.dtype == q.dtype), "softcap_attn: gate shape / format")
     t = q.shape[0]
     _need(q.shape == (t, heads * dim) and q.is_contiguous() and t == layout.n_tok, "softcap_attn: q must be contiguous (T, heads * dim)")
@@ -1092,8 +1096,9 @@ def softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, layout: Step
     lib = _lib.load()
     _lib.check(lib.nvx_softcap_attn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _fmt(q), _ptr(kv_indices), _ptr(kv_start), _ptr(kv_len),
                                     _ptr(layout.qo_indptr), _ptr(layout.tok_seq), float(scale), float(cap), _ptr(out), t, heads, kv_heads, dim,
-                                    vdim, n_split, _ptr(part), int(window or 0), _ptr(r1), _ptr(r2), _ptr(vfreq), int(bool(v_interleaved)),
-                                    _ptr(gate), gate.stride(0) if gate is not None else 0, _stream()), "nvx_softcap_attn")
+                                    vdim, n_split, _ptr(part), int(window or 0), _ptr(r1), _ptr(r2), _ptr(v_turn), int(bool(v_interleaved)),
+                                    _ptr(gate), gate.stride(0) if gate is not None else 0, layout.n_seq, int(bool(matrix_cores)), _stream()),
+               "nvx_softcap_attn")
     return out
 
 
@@ -1104,7 +1109,8 @@ def attn_prep_store(x, offsets, positions, q_w, k_w, norm_mode: str, eps: float,
     weights of heads * dim / kv_heads * dim entries; "none"), rotation of the first rot_dims of every q and k head by positions *
     freq (float64, rot_dims / 2; pairs (m, m + rot_dims / 2), or (2m, 2m + 1) if `interleaved`), rotation of every value head over
     all of vdim by positions * vfreq if vfreq is given, keys and values stored at k_cache[slots] / v_cache[slots].  With kv_heads
-    == 0 only the queries are prepared (k_w, slots and the caches may be None).  Returns the queries (T, heads * dim)."""
+    == 0 only the queries are prepared (k_w, slots and the caches may be None).  Returns (queries (T, heads * dim), v_turn): v_turn
+    (T, vdim) float32 holds every token's cos | sin of its value rotation (None without vfreq), for softcap_attn to turn back with."""
     _dev(x, positions, q_w, k_w, freq, vfreq, slots, k_cache, v_cache)
     t = x.shape[0]
     _need(x.dim() == 2 and x.stride(1) == 1, "attn_prep_store: x must be (T, columns) with unit inner stride")
@@ -1126,19 +1132,27 @@ def attn_prep_store(x, offsets, positions, q_w, k_w, norm_mode: str, eps: float,
         _need(k_cache.dtype == x.dtype and v_cache.dtype == x.dtype and k_cache.is_contiguous() and v_cache.is_contiguous() and
               k_cache.shape == (n_slots, kv_heads * dim) and v_cache.shape == (n_slots, kv_heads * vdim), "attn_prep_store: cache shapes")
     q = torch.empty((t, heads * dim), dtype=x.dtype, device=x.device)
+    v_turn = torch.empty((t, vdim), dtype=F32, device=x.device) if vfreq is not None else None
     lib = _lib.load()
     _lib.check(lib.nvx_attn_prep_store(_ptr(x), x.stride(0), _fmt(x), offsets[0], offsets[1], offsets[2], _ptr(positions), _ptr(q_w) if mode else None,
                                        _ptr(k_w) if mode and kv_heads else None, mode, float(eps), _ptr(freq) if rot_dims else None, rot_dims,
                                        int(bool(interleaved)), _ptr(vfreq), _ptr(slots) if kv_heads else None, _ptr(q),
                                        _ptr(k_cache) if kv_heads else None, _ptr(v_cache) if kv_heads else None, n_slots, t, heads, kv_heads, dim,
-                                       vdim, _stream()), "nvx_attn_prep_store")
-    return q
+                                       vdim, _ptr(v_turn), _stream()), "nvx_attn_prep_store")
+    return q, v_turn
 
 
-def decay_scan(x, offsets, decay, mem, layout: StepLayout, heads: int, dim: int, vdim: int, act: str = "none"):
+DECAY_SCAN_CHUNK = 128            # tokens of a chunk where long portions are cut into chunks that run side by side
+DECAY_SCAN_CHUNK_FROM = 512       # ... which pays from portions of this length on
+DECAY_SCAN_WS_BYTES = 1 << 30     # the chunks' states may take this much; longer chunks otherwise
+
+
+def decay_scan(x, offsets, decay, mem, layout: StepLayout, heads: int, dim: int, vdim: int, act: str = "none", chunk: Optional[int] = None):
     """Linear attention with one constant decay per head.  x (T, columns): q, k (heads * dim each) and v (heads * vdim) at the
     three column `offsets`, passed through `act` ("none" or "silu") first; decay (heads) float32; mem (slots, heads, dim, vdim)
-    float32, continued and written back.  S <- decay S + k v^T, read-out S^T q.  Returns (T, heads, vdim) float32."""
+    float32, continued and written back.  S <- decay S + k v^T, read-out S^T q.  Returns (T, heads, vdim) float32.
+    Ragged steps with long portions are cut into chunks of `chunk` tokens (default: by the step's shape; 0: never) that run side by
+    side: the result is the same up to the rounding of decay^n against n multiplications."""
     _dev(x, decay, mem)
     _need(x.dim() == 2 and x.stride(1) == 1 and x.shape[0] == layout.n_tok, "decay_scan: x must be (T, columns) with unit inner stride")
     _f32c(decay, "decay_scan: decay")
@@ -1147,10 +1161,22 @@ def decay_scan(x, offsets, decay, mem, layout: StepLayout, heads: int, dim: int,
     _need(decay.numel() == heads and mem.shape == (n_slots, heads, dim, vdim), "decay_scan: shapes")
     t = x.shape[0]
     out = torch.empty((t, heads, vdim), dtype=F32, device=x.device)
+    if chunk is None:
+        chunk = DECAY_SCAN_CHUNK if layout.qo_indptr is not None and layout.max_q >= DECAY_SCAN_CHUNK_FROM else 0
+    n_chunks, ws = 0, None
+    if chunk and layout.qo_indptr is not None:
+        per = heads * dim * vdim * 4
+        while layout.n_seq * -(-layout.max_q // chunk) * per > DECAY_SCAN_WS_BYTES or layout.n_seq * -(-layout.max_q // chunk) > 65535:
+            chunk *= 2
+        n_chunks = -(-layout.max_q // chunk)
+        if n_chunks > 1:
+            ws = torch.empty((layout.n_seq * n_chunks, heads, dim, vdim), dtype=F32, device=x.device)
+    if ws is None:
+        chunk = n_chunks = 0
     lib = _lib.load()
     _lib.check(lib.nvx_decay_scan(_ptr(x), x.stride(0), _fmt(x), offsets[0], offsets[1], offsets[2], {"none": 0, "silu": 1}[act], _ptr(decay),
-                                  _ptr(mem), n_slots, *_layout_args(layout), _ptr(out), t, layout.n_seq, heads, dim, vdim, _stream()),
-               "nvx_decay_scan")
+                                  _ptr(mem), n_slots, *_layout_args(layout), _ptr(out), t, layout.n_seq, heads, dim, vdim, chunk, n_chunks,
+                                  _ptr(ws), _stream()), "nvx_decay_scan")
     return out
 
 

@@ -84,11 +84,11 @@ _DEFS = {
                         "Tensor(b!) v_cache, int heads, int kv_heads, int dim, int vdim) -> Tensor",
     "softcap_attn": "(Tensor q, Tensor k_cache, Tensor v_cache, Tensor kv_indices, Tensor kv_start, Tensor kv_len, Tensor pos0, "
                     "Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq, float scale, float cap, int heads, int kv_heads, int dim, int vdim, "
-                    "int window=0, Tensor? r1=None, Tensor? r2=None, Tensor? vfreq=None, bool v_interleaved=False, Tensor? gate=None) -> Tensor",
+                    "int window=0, Tensor? r1=None, Tensor? r2=None, Tensor? v_turn=None, bool v_interleaved=False, Tensor? gate=None) -> Tensor",
     # post-normed stream, query/key norms with rotated values, decayed linear attention, experts with weights on their outputs
     "attn_prep_store": "(Tensor x, int q_off, int k_off, int v_off, Tensor positions, Tensor? q_w, Tensor? k_w, str norm_mode, float eps, "
                        "Tensor? freq, int rot_dims, bool interleaved, Tensor? vfreq, Tensor? slots, Tensor(a!)? k_cache, Tensor(b!)? v_cache, "
-                       "int heads, int kv_heads, int dim, int vdim) -> Tensor",
+                       "int heads, int kv_heads, int dim, int vdim) -> (Tensor, Tensor?)",
     "decay_scan": "(Tensor x, int q_off, int k_off, int v_off, Tensor decay, Tensor(a!) mem, Tensor pos0, Tensor state_slot, Tensor? qo_indptr, "
                   "Tensor? tok_seq, int heads, int dim, int vdim, str act) -> Tensor",
     "postnorm_residual": "(Tensor(a!) x, Tensor? y, Tensor? w_post, float eps, Tensor? y2, float a, float b, Tensor? w_next, ScalarType dtype) -> Tensor",
@@ -296,9 +296,9 @@ def _rope_vnorm_store(qkv, positions, freq, mag, rot_dims, eps, slots, k_cache, 
 
 
 def _softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, pos0, state_slot, qo_indptr, tok_seq, scale, cap, heads, kv_heads, dim, vdim,
-                  window=0, r1=None, r2=None, vfreq=None, v_interleaved=False, gate=None):
+                  window=0, r1=None, r2=None, v_turn=None, v_interleaved=False, gate=None):
     return ops.softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, _layout(q.shape[0], pos0, state_slot, qo_indptr, tok_seq), scale, cap,
-                            heads, kv_heads, dim, vdim, window=window, r1=r1, r2=r2, vfreq=vfreq, v_interleaved=v_interleaved, gate=gate)
+                            heads, kv_heads, dim, vdim, window=window, r1=r1, r2=r2, v_turn=v_turn, v_interleaved=v_interleaved, gate=gate)
 
 
 def _attn_prep_store(x, q_off, k_off, v_off, positions, q_w, k_w, norm_mode, eps, freq, rot_dims, interleaved, vfreq, slots, k_cache, v_cache,

@@ -104,8 +104,10 @@ def test_query_key_norms_rotation_and_rotated_values(mode, interleaved):
     qw, kw = (torch.randn(dim if mode == "head" else n, generator=g) for n in (nq, nk))
     freq, vfreq = rotary_frequencies(rot, base)[0], rotary_frequencies(vdim, base)[0]
     kc, vc = torch.full((8, nk), 9.0).cuda(), torch.full((8, nv), 9.0).cuda()
-    q = ops.attn_prep_store(x.cuda(), (5, 5 + nq, 5 + nq + nk), pos.cuda(), qw.cuda(), kw.cuda(), mode, 1e-4, freq.cuda(), rot, interleaved, vfreq.cuda(),
-                            slots.cuda(), kc, vc, heads, kvh, dim, vdim)
+    q, turn = ops.attn_prep_store(x.cuda(), (5, 5 + nq, 5 + nq + nk), pos.cuda(), qw.cuda(), kw.cuda(), mode, 1e-4, freq.cuda(), rot, interleaved,
+                                  vfreq.cuda(), slots.cuda(), kc, vc, heads, kvh, dim, vdim)
+    ang = pos.double()[:, None] * vfreq[None, :]
+    assert torch.allclose(turn.cpu().double(), torch.cat([torch.cos(ang), torch.sin(ang)], dim=1), atol=1e-6)
     xq, xk, xv = x[:, 5:5 + nq].double(), x[:, 5 + nq:5 + nq + nk].double(), x[:, 5 + nq + nk:5 + nq + nk + nv].double()
     if mode == "head":
         xq, xk = go.unit_rms(xq.view(t, heads, dim), 1e-4) * qw, go.unit_rms(xk.view(t, kvh, dim), 1e-4) * kw
@@ -122,9 +124,9 @@ def test_query_key_norms_rotation_and_rotated_values(mode, interleaved):
     untouched = [s for s in range(8) if s not in slots.tolist()]
     assert (kc.cpu()[untouched] == 9.0).all() and (vc.cpu()[untouched] == 9.0).all()
     # queries only: nothing is read or written for keys and values
-    q2 = ops.attn_prep_store(x.cuda(), (5, 0, 0), pos.cuda(), qw.cuda(), None, mode, 1e-4, freq.cuda(), rot, interleaved, None, None, None, None,
-                             heads, 0, dim, vdim)
-    assert torch.equal(q2, q)
+    q2, none = ops.attn_prep_store(x.cuda(), (5, 0, 0), pos.cuda(), qw.cuda(), None, mode, 1e-4, freq.cuda(), rot, interleaved, None, None, None, None,
+                                   heads, 0, dim, vdim)
+    assert torch.equal(q2, q) and none is None
 
 
 def _cached(keys, values, n_slots, seed):
@@ -140,8 +142,17 @@ def _cached(keys, values, n_slots, seed):
     return kc, vc, lists
 
 
-def _attend(ops, q_rows, lens, totals, lists, kc, vc, fmt, decode, **kw):
+def _turn_table(totals, lens, freq):
+    """cos | sin of position * freq for every token of a step, as attn_prep_store hands them to the attention."""
+    pos = torch.cat([torch.arange(n - l, n) for n, l in zip(totals, lens)]).double()
+    ang = pos[:, None] * freq.double().cpu()[None, :]
+    return torch.cat([torch.cos(ang), torch.sin(ang)], dim=1).float().cuda()
+
+
+def _attend(ops, q_rows, lens, totals, lists, kc, vc, fmt, decode, vfreq=None, **kw):
     """ops.softcap_attn for a step that brings the last lens[b] tokens of the first totals[b] of sequence b."""
+    if vfreq is not None:
+        kw["v_turn"] = _turn_table(totals, lens, vfreq)
     flat = torch.tensor([s for b, l in enumerate(lists) for s in l[:totals[b]]], dtype=torch.int32).cuda()
     start = torch.tensor(np.concatenate([[0], np.cumsum(totals)[:-1]]), dtype=torch.int64).cuda()
     kv_len = torch.tensor(totals, dtype=torch.int32).cuda()
@@ -187,6 +198,55 @@ def test_attention_window_and_distance_penalty(window, penalty):
     if window:
         wider = go.attend(q[0].double(), k[0].double(), v[0].double(), scale, cap=cap, window=window + 1, r1=r1, r2=r2)
         assert (wider[window:] - want[0][window:]).abs().max() > 0.1
+
+
+@pytest.mark.parametrize("dim,vdim", [(64, 96), (96, 64), (128, 128)])
+@pytest.mark.parametrize("window", [0, 5, 70])
+@pytest.mark.parametrize("interleaved", [False, True])
+def test_attention_on_the_matrix_cores(dim, vdim, window, interleaved):
+    """Steps of many tokens in bfloat16 take the tile kernel (64 queries of a sequence per workgroup, keys in tiles of 32): ragged
+    prompts that end in the middle of a tile, portions that start in the middle of one, a loud key just outside every window, the
+    distance penalty, the read-out turned back and gated; against the restatement on the same bfloat16 values, and against the
+    vector kernel."""
+    from nano_vllm_x_amd import ops
+    from nano_vllm_x_amd.layers.rotary_embedding import rotary_frequencies
+    g = torch.Generator().manual_seed(dim + window)
+    heads, kvh, scale, cap, base = 4, 2, 0.2, 9.0, 300.0
+    n = [200, 77, 300, 1]
+    bf = lambda x: x.to(torch.bfloat16).float()
+    q = [bf(torch.randn(t, heads, dim, generator=g)) for t in n]
+    k = [bf(torch.randn(t, kvh, dim, generator=g)) for t in n]
+    v = [bf(torch.randn(t, kvh, vdim, generator=g)) for t in n]
+    for b in range(len(n)):
+        for i in range(n[b]):
+            j = i - window if window and i >= window else 0
+            for h in range(heads):
+                kj = k[b][j, h // (heads // kvh)]
+                q[b][i, h] = bf(4.0 * kj / kj.norm())
+    gate = [bf(torch.randn(t, heads * vdim, generator=g)) for t in n]
+    r1, r2 = torch.tensor([0.9, 0.0, 0.3, 2.0]), torch.tensor([0.5, 3.0, 0.01, 1.0])
+    want = []
+    for b in range(len(n)):
+        pos = torch.arange(n[b])
+        turned = bf(go.turn(v[b].double(), pos, base, vdim, interleaved).float())            # values are cached turned, in bfloat16
+        v[b] = turned
+        o = go.attend(q[b].double(), k[b].double(), turned.double(), scale, cap=cap, window=window or None, r1=r1, r2=r2)
+        want.append(go.turn(o, pos, base, vdim, interleaved, sign=-1.0).reshape(n[b], -1) * torch.sigmoid(gate[b].double()))
+    kc, vc, lists = _cached(k, v, 700, 5)
+    vfreq = rotary_frequencies(vdim, base)[0].cuda()
+    kw = dict(scale=scale, cap=cap, heads=heads, kv_heads=kvh, dim=dim, vdim=vdim, window=window, r1=r1.cuda(), r2=r2.cuda(), vfreq=vfreq,
+              v_interleaved=interleaved, n_split=1)
+    assert ops._lib.load().nvx_softcap_attn_tile_fits(0, dim, vdim, int(not interleaved)) == 1
+    for lens, totals in ((n, n), ([70, 3, 130, 1], [200, 77, 300, 1]), ([129, 77, 1, 1], [130, 77, 65, 1])):
+        rows = torch.cat([q[b][totals[b] - lens[b]:totals[b]].reshape(lens[b], -1) for b in range(len(n))])
+        gates = torch.cat([gate[b][totals[b] - lens[b]:totals[b]] for b in range(len(n))]).to(torch.bfloat16).cuda()
+        ref = torch.cat([want[b][totals[b] - lens[b]:totals[b]] for b in range(len(n))])
+        tile = _attend(ops, rows, lens, totals, lists, kc, vc, torch.bfloat16, False, gate=gates, matrix_cores=True, **kw)
+        vec = _attend(ops, rows, lens, totals, lists, kc, vc, torch.bfloat16, False, gate=gates, matrix_cores=False, **kw)
+        for got, what in ((tile, "matrix cores"), (vec, "vector units")):
+            # results are bfloat16: half a unit in the last place is 2^-9 of the value; a wrong key would move them by tenths
+            err = ((got.double() - ref).abs() / (ref.abs() + 0.05 * ref.std())).max().item()
+            assert err < 8e-3, f"{what}, lens {lens} of {totals}: {err:.2e}"
 
 
 @pytest.mark.parametrize("interleaved", [False, True])
@@ -258,6 +318,39 @@ def test_decayed_memory_continues_over_cuts_and_reused_slots(dim, vdim):
     # the first token still counts at the end of the long sequence (heads with decay near one)
     other = ref(full[0][1:])
     assert (other[-1, 1:] - want[0][-1, 1:]).abs().max() > 1e-3
+
+
+@pytest.mark.parametrize("chunk", [16, 128, None])
+def test_decayed_memory_in_chunks_side_by_side(chunk):
+    """Long portions are cut into chunks that run side by side, the states at their starts carried between two launches: three
+    sequences of unequal length (one shorter than a chunk, one ending exactly at a chunk's edge), first from empty states, then
+    continued from the states the first step left; against the walk token by token of the restatement."""
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(3)
+    heads, dim, vdim = 3, 40, 24
+    decay = [0.7, 0.99, 1.0]
+    hd, he = heads * dim, heads * vdim
+    n1, n2 = [600, 9, 256], [530, 700, 1]
+    full = [torch.randn(a + b, 2 * hd + he, generator=g) * 0.5 for a, b in zip(n1, n2)]
+
+    def ref(x):
+        return go.decayed_memory(x[:, :hd].double().reshape(-1, heads, dim), x[:, hd:2 * hd].double().reshape(-1, heads, dim),
+                                 x[:, 2 * hd:].double().reshape(-1, heads, vdim), decay)
+    want = [ref(x) for x in full]
+    state = torch.full((4, heads, dim, vdim), 7.0).cuda()
+    dec = torch.tensor(decay).cuda()
+    slots = [2, 0, 3]
+    first = ops.decay_scan(torch.cat([x[:a] for x, a in zip(full, n1)]).cuda(), (0, hd, 2 * hd), dec, state,
+                           step_layout(ops, n1, [0, 0, 0], slots), heads, dim, vdim, chunk=chunk).cpu()
+    second = ops.decay_scan(torch.cat([x[a:] for x, a in zip(full, n1)]).cuda(), (0, hd, 2 * hd), dec, state,
+                            step_layout(ops, n2, n1, slots), heads, dim, vdim, chunk=chunk).cpu()
+    a1 = a2 = 0
+    for b in range(3):
+        close(first[a1:a1 + n1[b]], want[b][0][:n1[b]], 1e-4, f"sequence {b}, from an empty state")
+        close(second[a2:a2 + n2[b]], want[b][0][n1[b]:], 1e-4, f"sequence {b}, continued")
+        close(state[slots[b]].cpu(), want[b][1], 1e-4, f"sequence {b}, state left behind")
+        a1, a2 = a1 + n1[b], a2 + n2[b]
+    assert (state[1].cpu() == 7.0).all()
 
 
 @pytest.mark.parametrize("top,experts", [(1, 3), (2, 5), (3, 3)])
