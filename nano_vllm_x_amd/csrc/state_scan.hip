@@ -373,17 +373,20 @@ __global__ __launch_bounds__(256) void rwkv_scan_kernel(const A* __restrict__ rx
 // Because the decay is a constant, the carry over a chunk of n tokens is decay^n S + (the chunk's own contribution).  phase 0: one
 // workgroup walks the whole portion (single tokens, short portions).
 __device__ __forceinline__ float scan_act(float z, int act) { return act == 1 ? z * sigmoid_f(z) : z; }
-template <typename A>
+// `tb` tokens are staged at a time: 32 where the key size leaves LDS for them (more than the other recurrences take: an activation
+// is applied as they are staged, and fewer, longer stages hide more of the loads), fewer for wide keys.
+template <typename A, int PHASE>
 __global__ __launch_bounds__(256) void decay_scan_kernel(const A* __restrict__ x, int64_t x_stride, int q_off, int k_off, int v_off, int act,
                                                         const float* __restrict__ decay, float* __restrict__ S,
                                                         const int32_t* __restrict__ qo_indptr, const int64_t* __restrict__ pos0,
                                                         const int32_t* __restrict__ state_slot, float* __restrict__ out, int heads, int dim,
-                                                        int vdim, int p_lanes, int phase, int chunk, int n_chunk_max, float* __restrict__ ws) {
+                                                        int vdim, int p_lanes, int tb, int chunk, int n_chunk_max, float* __restrict__ ws) {
+    constexpr int phase = PHASE;
     extern __shared__ float sm[];
     const int cb = blockDim.x / p_lanes, rs = p_lanes * KS;
     float* sq = sm;
-    float* sk = sq + TB * rs;
-    float* sv = sk + TB * rs;
+    float* sk = sq + tb * rs;
+    float* sv = sk + tb * rs;
     const int hd = blockIdx.y;
     const int seq = phase ? blockIdx.z / n_chunk_max : blockIdx.z, ck = phase ? blockIdx.z % n_chunk_max : 0;
     SeqSpan sp = seq_span(seq, qo_indptr, pos0, state_slot);
@@ -404,15 +407,15 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(const A* __restrict__ x
         const int row = th.r0 + r;
         s[r] = (cont && row < dim && th.active) ? Sp[(int64_t)row * vdim + th.e] : 0.f;
     }
-    zero_rows(sq, 2 * TB * rs);
+    zero_rows(sq, 2 * tb * rs);
     const float g = decay[hd];
-    for (int64_t t0 = 0; t0 < sp.n; t0 += TB) {
-        const int nt = (int)(sp.n - t0 < TB ? sp.n - t0 : TB);
+    for (int64_t t0 = 0; t0 < sp.n; t0 += tb) {
+        const int nt = (int)(sp.n - t0 < tb ? sp.n - t0 : tb);
         __syncthreads();
         for (int i = threadIdx.x; i < nt * dim; i += blockDim.x) {
             const int tt = i / dim, d = i % dim;
             const int64_t r = (sp.q0 + t0 + tt) * x_stride + hd * dim + d;
-            sq[tt * rs + lds_row(d)] = scan_act(ld_f(x, r + q_off), act);
+            if (phase != 1) sq[tt * rs + lds_row(d)] = scan_act(ld_f(x, r + q_off), act);      // (phase 1 wants the state only)
             sk[tt * rs + lds_row(d)] = scan_act(ld_f(x, r + k_off), act);
         }
         for (int i = threadIdx.x; i < nt * cb; i += blockDim.x) {
@@ -425,13 +428,17 @@ __global__ __launch_bounds__(256) void decay_scan_kernel(const A* __restrict__ x
             const float v = sv[tt * cb + th.col];
             const float* kk = sk + tt * rs + th.p * KS;
             const float* qq = sq + tt * rs + th.p * KS;
+            if (phase == 1) {
+#pragma unroll
+                for (int r = 0; r < KR; ++r) s[r] = g * s[r] + kk[r] * v;
+                continue;
+            }
             float o = 0.f;
 #pragma unroll
             for (int r = 0; r < KR; ++r) {
                 s[r] = g * s[r] + kk[r] * v;
                 o += s[r] * qq[r];
             }
-            if (phase == 1) continue;                // (only the state is wanted)
             o = lanes_sum(o, p_lanes);
             if (th.p == 0 && th.active) out[(sp.q0 + t0 + tt) * (int64_t)heads * vdim + (int64_t)hd * vdim + th.e] = o;
         }
@@ -611,14 +618,15 @@ extern "C" int nvx_decay_scan(const void* x, int64_t x_stride, int fmt, int64_t 
     NVX_REQUIRE(x && decay && S && out, NVX_EINVAL, "nvx_decay_scan: null pointer");
     NVX_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && x_stride >= q_off + heads * dim && x_stride >= k_off + heads * dim &&
                     x_stride >= v_off + heads * vdim, NVX_EINVAL, "nvx_decay_scan: q, k or v lies outside a row");
-    const size_t lds = (size_t)(2 * TB * g.p_lanes * KS + TB * g.cb) * sizeof(float);
+    const int tb = g.p_lanes <= 4 ? 32 : (g.p_lanes == 8 ? 16 : TB);
+    const size_t lds = (size_t)(2 * tb * g.p_lanes * KS + tb * g.cb) * sizeof(float);
     NVX_REQUIRE(chunk == 0 || (chunk > 0 && chunk < (1 << 30) && n_chunk_max > 0 && n_seq * n_chunk_max <= 65535 && ws && qo_indptr), NVX_EINVAL,
                 "nvx_decay_scan: chunks need a ragged step, their workspace, and at most 65535 of them");
     const dim3 grid((unsigned)((vdim + g.cb - 1) / g.cb), (unsigned)heads, (unsigned)(chunk ? n_seq * n_chunk_max : n_seq));
 #define NVX_DECAY_SCAN(PHASE)                                                                                                                      \
-    NVX_FMT_CALL(fmt, hipLaunchKernelGGL(decay_scan_kernel<A_>, grid, dim3(g.threads), lds, (hipStream_t)stream, (const A_*)x, x_stride, (int)q_off, \
-                                         (int)k_off, (int)v_off, act, decay, S, qo_indptr, pos0, state_slot, out, (int)heads, (int)dim, (int)vdim, \
-                                         g.p_lanes, PHASE, (int)chunk, (int)n_chunk_max, ws))
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL((decay_scan_kernel<A_, PHASE>), grid, dim3(g.threads), lds, (hipStream_t)stream, (const A_*)x, x_stride,   \
+                                         (int)q_off, (int)k_off, (int)v_off, act, decay, S, qo_indptr, pos0, state_slot, out, (int)heads, (int)dim,  \
+                                         (int)vdim, g.p_lanes, tb, (int)chunk, (int)n_chunk_max, ws))
     if (!chunk) {
         NVX_DECAY_SCAN(0);
     } else {

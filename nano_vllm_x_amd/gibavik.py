@@ -244,6 +244,8 @@ class GibavikForCausalLM(nn.Module):
         n_layers = len(self.layers)
         if n_layers == 0:
             return ops.postnorm_residual(x, w_next=self.final_norm, eps=eps, out_dtype=self.embed.dtype)
+        # the experts of a token hang on its id alone: every layer's choices and expert order are made now, with one host read
+        plans = TableMoE.plan_step([l.mlp if l.mlp_kind == "moe" else None for l in self.layers], input_ids, decode_step)
         for i, layer in enumerate(self.layers):
             last = i + 1 == n_layers
             closing = self.final_norm if last and layer.mlp is None else None
@@ -255,7 +257,7 @@ class GibavikForCausalLM(nn.Module):
             else:
                 h = ops.postnorm_residual(x, y=layer.mixer(h, positions, md), w_post=layer.norm1, eps=eps, w_next=closing)
             if layer.mlp is not None:
-                y = layer.mlp(h) if layer.mlp_kind == "dense" else layer.mlp(h, input_ids, decode_step)
+                y = layer.mlp(h) if layer.mlp_kind == "dense" else layer.mlp(h, input_ids, decode_step, plan=plans[i])
                 h = ops.postnorm_residual(x, y=y, w_post=layer.norm2, eps=eps, w_next=self.final_norm if last else None)
             if self.layer_streams is not None:
                 self.layer_streams.append(x.clone())

@@ -30,17 +30,25 @@ class ExpertBank(nn.Module):
         self.w_d = nn.Parameter(torch.empty(experts, width, ff))
         self._rows_fit = None
 
-    def run(self, h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, decode_step: bool, weight_out: bool) -> torch.Tensor:
-        t = h.shape[0]
+    def by_rows(self, t: int, decode_step: bool) -> bool:
+        """Whether a step of t tokens streams the chosen experts' rows (else: per-expert products over the expert order)."""
         if self._rows_fit is None:
             self._rows_fit = ops.moe_expert_rows_fits(self.width, self.ff)
             self._order_fit = ops.moe_order_fits(self.experts)      # more experts than the ordering kernel holds: pair by pair
             if not (self._rows_fit or self._order_fit):
                 raise NotImplementedError(f"{self.experts} experts of {self.ff} x {self.width}: neither expert path is built for these sizes")
-        if self._rows_fit and (decode_step or t <= self.ROWS_PATH_TOKENS or not self._order_fit):
+        return self._rows_fit and (decode_step or t <= self.ROWS_PATH_TOKENS or not self._order_fit)
+
+    def run(self, h: torch.Tensor, idx: torch.Tensor, wts: torch.Tensor, decode_step: bool, weight_out: bool, order=None) -> torch.Tensor:
+        """`order` = (dst, counts as a list): the expert order of idx where the caller has it already (ops.moe_order)."""
+        t = h.shape[0]
+        if self.by_rows(t, decode_step):
             return ops.moe_expert_rows(h, idx, wts, self.w_gu, self.w_d, self.limit, self.alpha, self.shift, weight_out)
-        dst, counts = ops.moe_order(idx, self.experts)
-        counts = counts.tolist()
+        if order is None:
+            dst, counts = ops.moe_order(idx, self.experts)
+            counts = counts.tolist()
+        else:
+            dst, counts = order
         xs = ops.moe_scatter_rows(h, None if weight_out else wts, dst)
         gu = torch.empty((xs.shape[0], 2 * self.ff), dtype=h.dtype, device=h.device)
         a = 0
@@ -81,7 +89,37 @@ class TableMoE(ExpertBank):
         self.register_buffer("table", torch.zeros(vocab, top, dtype=torch.int32), persistent=False)
         self.register_buffer("share", torch.full((1, top), 1.0 / top, dtype=torch.float32), persistent=False)
 
-    def forward(self, h: torch.Tensor, input_ids: torch.Tensor, decode_step: bool = False) -> torch.Tensor:
+    def choices(self, input_ids: torch.Tensor):
+        """(idx, wts) of a step's tokens: they depend on the token ids alone."""
         idx = self.table.index_select(0, input_ids)
-        wts = self.share.expand(idx.shape[0], self.top).contiguous()
-        return self.run(h, idx, wts, decode_step, weight_out=True)
+        return idx, self.share.expand(idx.shape[0], self.top).contiguous()
+
+    @staticmethod
+    def plan_step(layers, input_ids: torch.Tensor, decode_step: bool) -> list:
+        """What every TableMoE of `layers` (None where a layer has none) needs for this step, made before the first layer runs: the
+        choices, and for steps of many tokens the expert order with its counts -- ONE host read for all layers instead of one per
+        layer in the middle of the step, so the host can queue the whole step without waiting for the device."""
+        plans, pending = [], []
+        for moe in layers:
+            if moe is None:
+                plans.append(None)
+                continue
+            idx, wts = moe.choices(input_ids)
+            plan = {"idx": idx, "wts": wts, "order": None}
+            if not moe.by_rows(idx.shape[0], decode_step):
+                dst, counts = ops.moe_order(idx, moe.experts)
+                pending.append((plan, dst, counts))
+            plans.append(plan)
+        if pending:
+            flat = torch.cat([c for _, _, c in pending]).tolist()
+            at = 0
+            for plan, dst, counts in pending:
+                plan["order"] = (dst, flat[at:at + counts.numel()])
+                at += counts.numel()
+        return plans
+
+    def forward(self, h: torch.Tensor, input_ids: torch.Tensor, decode_step: bool = False, plan=None) -> torch.Tensor:
+        if plan is None:
+            idx, wts = self.choices(input_ids)
+            return self.run(h, idx, wts, decode_step, weight_out=True)
+        return self.run(h, plan["idx"], plan["wts"], decode_step, weight_out=True, order=plan["order"])
