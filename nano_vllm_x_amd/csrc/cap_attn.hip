@@ -55,6 +55,15 @@ __global__ __launch_bounds__(256) void rope_vnorm_store_kernel(const A* __restri
 }
 
 
+// cos and sin of an angle given in double precision (position * frequency, exact to the table's accuracy at any position): the
+// angle is brought into [-pi, pi] in double precision, where its float32 value is off by at most 2e-7, and the float32 functions
+// take it from there.
+__device__ __forceinline__ void turn_of(double a, float& c, float& s) {
+    const double two_pi = 6.283185307179586476925286766559;
+    const float r = (float)(a - two_pi * rint(a / two_pi));
+    sincosf(r, &s, &c);
+}
+
 // One workgroup per token.  q, k and v are heads * dim, kv_heads * dim and kv_heads * vdim elements of row t of x, at q_off, k_off
 // and v_off (kv_heads == 0: a layer that borrows another layer's keys and values prepares its queries only).
 //   norm_mode 1: every query and key head is divided by its root mean square and multiplied by q_w / k_w (dim entries, shared by
@@ -62,7 +71,7 @@ __global__ __launch_bounds__(256) void rope_vnorm_store_kernel(const A* __restri
 //                heads * dim / kv_heads * dim entries;  0: no norm.
 //   The first rot_dims of every q and k head are then turned in pairs by positions[t] * freq[m]: pair m is (m, m + rot_dims / 2), or
 //   (2m, 2m + 1) if `interleaved`.  With vfreq, every value head is turned the same way over all of vdim by positions[t] * vfreq[m].
-// Angles, cosines and sines are formed in double precision; the norm is float32.  vcs_out (n_tok, vdim), if given, receives every
+// Angles are formed and reduced in double precision, cosines and sines taken in float32 from the reduced angle; the norm is float32.  vcs_out (n_tok, vdim), if given, receives every
 // token's cos | sin of positions[t] * vfreq[m] (vdim / 2 each).
 template <typename A>
 __global__ __launch_bounds__(256) void attn_prep_store_kernel(const A* __restrict__ x, int64_t x_stride, int q_off, int k_off, int v_off,
@@ -82,15 +91,11 @@ __global__ __launch_bounds__(256) void attn_prep_store_kernel(const A* __restric
     const int64_t t = blockIdx.x;
     const double pos = (double)positions[t];
     const A* row = x + t * x_stride;
-    for (int i = threadIdx.x; i < half; i += 256) {
-        const double a = pos * freq[i];
-        cs[i] = (float)cos(a);
-        cs[half + i] = (float)sin(a);
-    }
+    for (int i = threadIdx.x; i < half; i += 256) turn_of(pos * freq[i], cs[i], cs[half + i]);
     if (vfreq)                          // also handed out (vcs_out[t] = cos | sin): the attention turns its read-out back by the same angles
         for (int i = threadIdx.x; i < vhalf; i += 256) {
-            const double a = pos * vfreq[i];
-            const float cv = (float)cos(a), sv = (float)sin(a);
+            float cv, sv;
+            turn_of(pos * vfreq[i], cv, sv);
             vcs[i] = cv;
             vcs[vhalf + i] = sv;
             if (vcs_out) { vcs_out[t * (int64_t)vdim + i] = cv; vcs_out[t * (int64_t)vdim + vhalf + i] = sv; }
@@ -367,10 +372,13 @@ __global__ __launch_bounds__(256) void softcap_attn_tile_kernel(const A* __restr
     __shared__ A vt_lds[vdim * VT_ROW];
     __shared__ int where[2];
     if (threadIdx.x == 0) {          // which sequence and which block of its tokens: sequences take ceil(tokens / 64) workgroups each
-        int rem = blockIdx.x, found = -1;
-        for (int b = 0; b < n_seq; ++b) {
+        // Workgroups start in the order of their numbers, and a block late in a portion has the most keys to walk: the count runs
+        // backwards (last sequence first, and of a sequence its last block first), all heads of a block side by side, so the long
+        // walks start first and the short ones fill the end.
+        int rem = (int)(gridDim.y - 1 - blockIdx.y), found = -1;
+        for (int b = n_seq - 1; b >= 0; --b) {
             const int nb = (qo_indptr[b + 1] - qo_indptr[b] + TILE_Q - 1) / TILE_Q;
-            if (rem < nb) { found = b; break; }
+            if (rem < nb) { found = b; rem = nb - 1 - rem; break; }
             rem -= nb;
         }
         where[0] = found;
@@ -379,7 +387,7 @@ __global__ __launch_bounds__(256) void softcap_attn_tile_kernel(const A* __restr
     __syncthreads();
     const int b = where[0];
     if (b < 0) return;               // (the grid is an upper bound)
-    const int hd = blockIdx.y, kvh = hd / (heads / kv_heads);
+    const int hd = blockIdx.x, kvh = hd / (heads / kv_heads);
     const int q0 = qo_indptr[b], q_n = qo_indptr[b + 1] - q0, qs = where[1] * TILE_Q;
     const int rows_here = q_n - qs < TILE_Q ? q_n - qs : TILE_Q;
     const int pos_first = kv_len[b] - q_n + qs;                 // position of the block's first query
@@ -420,25 +428,34 @@ __global__ __launch_bounds__(256) void softcap_attn_tile_kernel(const A* __restr
 #pragma unroll
         for (int u = 0; u < VPT; ++u) { const int j = j0 + ((threadIdx.x + 256 * u) & (TILE_K - 1)); v_slot[u] = slots[j < hi ? j : hi - 1]; }
     };
-    auto fetch_rows = [&]() {
-        if (wave_on) {
+    auto fetch_key_rows = [&]() {
 #pragma unroll
-            for (int hh = 0; hh < 2; ++hh) {
-                const A* kr = k_cache + (int64_t)k_slot[hh] * k_row + (int64_t)kvh * dim + 8 * g;
+        for (int hh = 0; hh < 2; ++hh) {
+            const A* kr = k_cache + (int64_t)k_slot[hh] * k_row + (int64_t)kvh * dim + 8 * g;
 #pragma unroll
-                for (int s = 0; s < DS; ++s) kf[hh][s] = *reinterpret_cast<const nvx_u32x4*>(kr + 32 * s);
-            }
+            for (int s = 0; s < DS; ++s) kf[hh][s] = *reinterpret_cast<const nvx_u32x4*>(kr + 32 * s);
         }
+    };
+    auto fetch_value_rows = [&]() {
 #pragma unroll
         for (int u = 0; u < VPT; ++u) {
             const int i = threadIdx.x + 256 * u;
             if (i < VCH) vf[u] = *reinterpret_cast<const vec8*>(v_cache + (int64_t)v_slot[u] * v_row + (int64_t)kvh * vdim + (i / TILE_K) * 8);
         }
     };
+    // Scores live in the log2 domain (the hardware's exponential and logarithm are base 2): s2 = log2(e) * score.
+    //   no cap:  s2 = acc * (scale log2 e);   cap:  tanh(x) = 1 - 2 / (e^(2x) + 1), so s2 = (cap log2 e) (1 - 2 / (2^(acc * 2 scale log2 e / cap) + 1));
+    //   penalty: s2 -= r1 log2(1 + r2 distance).
+    constexpr float LOG2E = 1.4426950408889634f;
+    const float k_lin = cap > 0.f ? 2.0f * scale * LOG2E / cap : scale * LOG2E, k_cap = cap * LOG2E;
     const int j_begin = lo & ~(TILE_K - 1);
     fetch_slots(j_begin);
-    fetch_rows();
+    if (wave_on) fetch_key_rows();
+    fetch_value_rows();
     if (j_begin + TILE_K < hi) fetch_slots(j_begin + TILE_K);
+    const int q_lo = pos_first + wave * 16;                          // positions of this wave's first and last query
+    const int q_hi = q_lo + 15;
+    const bool rows_full = wave * 16 + 16 <= rows_here;
     for (int j0 = j_begin; j0 < hi; j0 += TILE_K) {
         __syncthreads();                                             // the tile before has been read by all waves
 #pragma unroll
@@ -450,31 +467,39 @@ __global__ __launch_bounds__(256) void softcap_attn_tile_kernel(const A* __restr
                 for (int e = 0; e < 8; ++e) vt_lds[(ch * 8 + e) * VT_ROW + kk] = vf[u][e];
             }
         }
-        nvx_u32x4 kc[2][DS];
-#pragma unroll
-        for (int hh = 0; hh < 2; ++hh)
-#pragma unroll
-            for (int s = 0; s < DS; ++s) kc[hh][s] = kf[hh][s];
-        if (j0 + TILE_K < hi) fetch_rows();                          // (with the ids read one step ago)
-        if (j0 + 2 * TILE_K < hi) fetch_slots(j0 + 2 * TILE_K);
         __syncthreads();
-        if (!wave_on) continue;
-        if (j0 >= w_hi || j0 + TILE_K <= w_lo) continue;            // none of this wave's queries sees the tile
+        // issued behind the barrier (which waits for every load before it): the next tile's rows and the ids of the one after
+        // travel while this tile's products run; the key rows as soon as this tile's have been multiplied
+        const bool more = j0 + TILE_K < hi;
+        if (more) fetch_value_rows();                                // (with the ids read one step ago)
+        if (!wave_on) {
+            if (j0 + 2 * TILE_K < hi) fetch_slots(j0 + 2 * TILE_K);
+            continue;
+        }
+        const bool seen = j0 < w_hi && j0 + TILE_K > w_lo;           // some query of this wave sees some key of the tile
+        nvx_f32x4 sacc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        if (seen) {
+#pragma unroll
+            for (int s = 0; s < DS; ++s) {
+                sacc[0] = ca_mfma32<A>(kf[0][s], qb[s], sacc[0]);
+                sacc[1] = ca_mfma32<A>(kf[1][s], qb[s], sacc[1]);
+            }
+        }
+        if (more) fetch_key_rows();
+        if (j0 + 2 * TILE_K < hi) fetch_slots(j0 + 2 * TILE_K);
+        if (!seen) continue;
+        // every query of the wave sees every key of the tile (most tiles): no mask to work out
+        const bool full = rows_full && j0 + TILE_K - 1 <= q_lo && (window <= 0 || j0 > q_hi - window);
         float sv[8], mx = -INFINITY;
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
-            nvx_f32x4 sacc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < DS; ++s) sacc = ca_mfma32<A>(kc[hh][s], qb[s], sacc);
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int j = j0 + hh * 16 + 4 * g + r;
-                float sc = -INFINITY;
-                if (row_on && j <= pos && (window <= 0 || j > pos - window)) {
-                    sc = sacc[r] * scale;
-                    if (cap > 0.f) sc = cap * (1.0f - 2.0f / (__expf(2.0f * sc / cap) + 1.0f));      // tanh by the hardware exponential
-                    if (r1) sc -= pen_a * __logf(1.0f + pen_b * (float)(pos - j));
-                }
+                float sc = sacc[hh][r] * k_lin;
+                if (cap > 0.f) sc = k_cap - 2.0f * k_cap * __builtin_amdgcn_rcpf(__builtin_amdgcn_exp2f(sc) + 1.0f);
+                if (r1) sc -= pen_a * __builtin_amdgcn_logf(1.0f + pen_b * (float)(pos - j));
+                if (!full && !(row_on && j <= pos && (window <= 0 || j > pos - window))) sc = -INFINITY;
                 sv[hh * 4 + r] = sc;
                 mx = fmaxf(mx, sc);
             }
@@ -482,13 +507,14 @@ __global__ __launch_bounds__(256) void softcap_attn_tile_kernel(const A* __restr
         mx = fmaxf(mx, xor16(mx));
         mx = fmaxf(mx, xor32(mx));
         const float m_new = fmaxf(m_run, mx);
-        const float alpha = m_new == -INFINITY ? 1.0f : __expf(m_run - m_new);    // (nothing seen yet: nothing to rescale)
+        const float alpha = m_new == -INFINITY ? 1.0f : __builtin_amdgcn_exp2f(m_run - m_new);    // (nothing seen yet: nothing to rescale)
         m_run = m_new;
         l_run *= alpha;
+        const float m_sub = m_new == -INFINITY ? 0.f : m_new;        // (then every score is -inf and every weight 0)
         float p[8], ph[8];
 #pragma unroll
         for (int e = 0; e < 8; ++e) {
-            p[e] = sv[e] == -INFINITY ? 0.f : __expf(sv[e] - m_new);
+            p[e] = __builtin_amdgcn_exp2f(sv[e] - m_sub);
             l_run += p[e];
             ph[e] = (float)(A)p[e];
         }
@@ -667,7 +693,8 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
     if (matrix_cores && nvx_softcap_attn_tile_fits(fmt, dim, vdim, vcs != nullptr && !v_interleaved) && qo_indptr && n_split == 1 && n_seq > 0 &&
         nvx_aligned16(q) && nvx_aligned16(k_cache) && nvx_aligned16(v_cache) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0 &&
         (!gate || ((reinterpret_cast<uintptr_t>(gate) & 7u) == 0 && gate_stride % 4 == 0))) {
-        const dim3 tgrid((unsigned)((n_tok + TILE_Q - 1) / TILE_Q + n_seq), (unsigned)heads);
+        NVX_REQUIRE((n_tok + TILE_Q - 1) / TILE_Q + n_seq <= 65535, NVX_EINVAL, "nvx_softcap_attn: too many tokens or sequences in one step");
+        const dim3 tgrid((unsigned)heads, (unsigned)((n_tok + TILE_Q - 1) / TILE_Q + n_seq));
 #define NVX_TILE_ATTN(DS, VT)                                                                                                            \
     NVX_FMT_CALL(fmt, hipLaunchKernelGGL((softcap_attn_tile_kernel<typename tile_fmt<A_>::type, DS, VT>), tgrid, dim3(256), 0, (hipStream_t)stream, \
                                          (const typename tile_fmt<A_>::type*)q, (const typename tile_fmt<A_>::type*)k_cache,            \

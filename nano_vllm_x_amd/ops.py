@@ -1142,8 +1142,10 @@ def attn_prep_store(x, offsets, positions, q_w, k_w, norm_mode: str, eps: float,
     return q, v_turn
 
 
-DECAY_SCAN_CHUNK = 128            # tokens of a chunk where long portions are cut into chunks that run side by side
-DECAY_SCAN_CHUNK_FROM = 512       # ... which pays from portions of this length on
+DECAY_SCAN_CHUNK_FROM = 256       # portions from this length on are cut into chunks that run side by side
+DECAY_SCAN_CHUNKS = ((65536, 32), (131072, 64), (None, 128))      # (tokens x heads of a step up to ..., tokens of a chunk): short chunks while
+# the step is too small to fill the chip with long ones, long chunks (fewer carried states) from there on (4 x 1 024 tokens, 8
+# heads: 895 us in one walk, 301 in chunks of 128, 150 in chunks of 32; 16 x 1 024 tokens: 446 us at 128 and 64, 474 at 32)
 DECAY_SCAN_WS_BYTES = 1 << 30     # the chunks' states may take this much; longer chunks otherwise
 
 
@@ -1162,7 +1164,9 @@ def decay_scan(x, offsets, decay, mem, layout: StepLayout, heads: int, dim: int,
     t = x.shape[0]
     out = torch.empty((t, heads, vdim), dtype=F32, device=x.device)
     if chunk is None:
-        chunk = DECAY_SCAN_CHUNK if layout.qo_indptr is not None and layout.max_q >= DECAY_SCAN_CHUNK_FROM else 0
+        chunk = 0
+        if layout.qo_indptr is not None and layout.max_q >= DECAY_SCAN_CHUNK_FROM:
+            chunk = next(c for upto, c in DECAY_SCAN_CHUNKS if upto is None or t * heads <= upto)
     n_chunks, ws = 0, None
     if chunk and layout.qo_indptr is not None:
         per = heads * dim * vdim * 4
