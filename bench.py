@@ -651,9 +651,9 @@ def _gibavik_config(z):
     moe = {"kind": "moe", "expert": {"ff": z["ff"] // 2}, "router": {"experts": 8, "top": 2}}
     dense = {"kind": "dense", "ff": z["ff"], "limit": 7.0}
     par = {"type": "parallel", "mixer": {
-        "left": {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 50.0, "mask": {"size": 512},
-                 "rot": {"dims": 64, "base": 1e6}},
-        "right": {"heads": hd, "dim": 64, "vdim": 128, "decay": [1.0 - 2.0 ** -(3 + j % 8) for j in range(hd)]}, "left_scale": 0.6, "right_scale": 1.1}}
+        "left": {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0, "mask": {"size": 512},
+                 "rot": {"dims": 64, "base": 5e5}},
+        "right": {"heads": hd, "dim": 64, "vdim": 128, "decay": [1.0 - 2.0 ** -(3 + j % 8) for j in range(hd)]}, "left_scale": 0.5, "right_scale": 1.0}}
     att = {"type": "attention", "mixer": {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5}}
     layers = []
     for i in range(z["layers"]):
@@ -704,7 +704,7 @@ def _gibavik_kernel_table(z, t_pre, n_dec, ctx, phases=("prefill", "decode")):
         # sublayer boundary: reads the result (2 B; two of them after a parallel mixer) and the stream (4 B), writes the stream (4 B) and
         # the rows the next sublayer reads (2 B)
         add("postnorm_residual", phase, _time_us(lambda: ops.postnorm_residual(x, y=y, w_post=one, eps=1e-5)), bytes_=t * w * 12, like="rmsnorm+residual")
-        add("postnorm_residual, two results", phase, _time_us(lambda: ops.postnorm_residual(x, y=y, y2=y2, a=0.6, b=1.1, w_post=one, eps=1e-5)),
+        add("postnorm_residual, two results", phase, _time_us(lambda: ops.postnorm_residual(x, y=y, y2=y2, a=0.5, b=1.0, w_post=one, eps=1e-5)),
             bytes_=t * w * 14, like="gated_residual_norm")
         xb = x.to(bf)
         add("qwen3 rmsnorm+residual", phase, _time_us(lambda: ops.rmsnorm(y, wv.to(bf), 1e-5, xb)), bytes_=t * w * 8)
@@ -748,7 +748,7 @@ def _gibavik_kernel_table(z, t_pre, n_dec, ctx, phases=("prefill", "decode")):
         qkv = torch.randn(t, (h + 16) * 128 + h * 128, device=dev).to(bf)          # q | k | v | g
         pos = (torch.arange(t, device=dev) % q_len + pos0).to(torch.int64)
         slots = (torch.arange(t, device=dev) // q_len * kv_len + pos).to(torch.int64)
-        fr, vfr = rotary_frequencies(64, 1e6)[0].to(dev), rotary_frequencies(128, 1e6)[0].to(dev)
+        fr, vfr = rotary_frequencies(64, 5e5)[0].to(dev), rotary_frequencies(128, 5e5)[0].to(dev)
         qn = torch.ones(128, device=dev)
         prep_bytes = t * (h + 16) * 128 * 2 * 2
         add("attn_prep_store (head norms, rotation, rotated values)", phase,
@@ -768,7 +768,7 @@ def _gibavik_kernel_table(z, t_pre, n_dec, ctx, phases=("prefill", "decode")):
         g128 = qkv[:, (h + 16) * 128:]
         vturn = torch.randn(t, 128, device=dev)
         r1, r2 = torch.full((h,), 0.5, device=dev), torch.full((h,), 0.1, device=dev)
-        us_win = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 50.0, h, 8, 128, 128, window=window, v_turn=vturn, gate=g128), reps)
+        us_win = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 30.0, h, 8, 128, 128, window=window, v_turn=vturn, gate=g128), reps)
         us_pen = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 0.0, h, 8, 128, 128, r1=r1, r2=r2), reps)
         us_plain = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 30.0, h, 8, 128, 128), reps)
         kc4, vc4 = kc.view(n_rows, 8, 128), vc.view(n_rows, 8, 128)

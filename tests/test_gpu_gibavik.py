@@ -65,8 +65,8 @@ def test_normed_results_are_added_to_the_stream(fmt, width):
     assert torch.allclose(xd.cpu(), want, atol=1e-5) and h.dtype == fmt and torch.allclose(h.float().cpu(), want, atol=tol)
     # two results weighted and summed before the norm, a weight per channel, and the closing norm on the new stream
     xd = x.cuda()
-    h = ops.postnorm_residual(xd, y=y.cuda(), y2=y2.cuda(), a=0.6, b=1.1, w_post=per.cuda(), eps=1e-3, w_next=nxt.cuda())
-    want = x + go.unit_rms(0.6 * y.float() + 1.1 * y2.float(), 1e-3) * per
+    h = ops.postnorm_residual(xd, y=y.cuda(), y2=y2.cuda(), a=0.7, b=1.3, w_post=per.cuda(), eps=1e-3, w_next=nxt.cuda())
+    want = x + go.unit_rms(0.7 * y.float() + 1.3 * y2.float(), 1e-3) * per
     assert torch.allclose(xd.cpu(), want, atol=1e-5) and torch.allclose(h.float().cpu(), go.scalar_norm(want, nxt, 1e-3), atol=tol)
     # the closing norm alone leaves the stream as it is
     xd = x.cuda()
@@ -84,7 +84,7 @@ def test_scaled_embedding_and_capped_logits():
         assert x.dtype == torch.float32 and h.dtype == fmt
         assert torch.equal(x.cpu(), table.to(fmt).float()[ids] * 12.5) and torch.equal(h.cpu(), (table.to(fmt).float()[ids] * 12.5).to(fmt))
     z = torch.randn(4, 70, generator=g) * 30
-    assert torch.allclose(ops.tanh_cap(z.cuda(), 15.0).cpu(), 15.0 * torch.tanh(z / 15.0), atol=1e-5)
+    assert torch.allclose(ops.tanh_cap(z.cuda(), 11.0).cpu(), 11.0 * torch.tanh(z / 11.0), atol=1e-5)
     assert torch.equal(ops.tanh_cap(z.to(torch.bfloat16).cuda(), 0.0).cpu(), z.to(torch.bfloat16).float())
 
 
@@ -281,7 +281,7 @@ def test_decayed_memory_continues_over_cuts_and_reused_slots(dim, vdim):
     from nano_vllm_x_amd import ops
     g = torch.Generator().manual_seed(dim)
     heads = 3
-    decay = [0.6, 0.999, 1.0]
+    decay = [0.6, 0.9975, 1.0]
     hd, he = heads * dim, heads * vdim
     full = {0: torch.randn(130, 2 + 2 * hd + he, generator=g), 1: torch.randn(17, 2 + 2 * hd + he, generator=g), 2: torch.randn(9, 2 + 2 * hd + he, generator=g)}
     silu = torch.nn.functional.silu
