@@ -176,7 +176,7 @@ def forward(cfg: dict, p: dict, tokens, dtype=F64, streams=None):
     eps = float(cfg["norm"]["eps"])
     tokens = torch.as_tensor(tokens, dtype=torch.int64)
     pos = torch.arange(len(tokens))
-    x = p["embed"].to(dtype)[tokens] * float(cfg["embedding"]["scale"])
+    x = p["embed"].to(dtype)[tokens] * float((cfg.get("embedding") or {}).get("scale", 1.0))
     kept = {}
     for i, spec in enumerate(cfg["layers"]):
         pre, m = f"l{i}.mix.", spec["mixer"]

@@ -407,6 +407,32 @@ def test_each_mixer_alone_whole_cut_and_token_by_token(tmp_path, name):
     eng.shutdown()
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_that_fit_no_vector_width(tmp_path, dtype):
+    """A width, head sizes, feed-forward sizes and a vocabulary that are multiples of nothing useful (no 16-byte rows anywhere), three
+    query heads on one key/value head, experts in the first layer and a dense feed-forward in the last."""
+    odd = [{"type": "attention", "mixer": {"heads": 3, "kv_heads": 1, "dim": 10, "vdim": 6, "scale": 0.3}, "mlp": {"kind": "moe", "expert": {"ff": 9}, "router": {"experts": 4, "top": 3}}},
+           _par(left={"heads": 3, "kv_heads": 3, "dim": 6, "vdim": 10, "mask": {"size": 4}, "rot": {"dims": 4, "base": 77.0}, "softcap": None},
+                right={"heads": 2, "dim": 5, "vdim": 7, "decay": [0.3, 0.97]}, mlp=None),
+           borrowing({"mixer": {"heads": 1, "kv_heads": 1, "dim": 10, "vdim": 6, "scale": 1.0}}, 0, {"kind": "dense", "ff": 11, "limit": 0.7})]
+    odd[1]["mixer"]["left"].pop("softcap")
+    cfg = make_cfg(odd, width=50, vocab=37, emb=1.0, cap=0.0)
+    cfg.pop("logit_softcap")
+    cfg.pop("embedding")
+    w = weights_of(cfg, 4)
+    eng = make_engine(model_dir(tmp_path, cfg, w), dtype=dtype, pool=256)
+    toks = tokens(45, 37, 8)
+    want = forward(cfg, w, toks)
+    got = replay(eng, {"a": toks}, [[("a", 33)], [("a", 2)]] + [[("a", 1)]] * 10)["a"]
+    if dtype == "float32":
+        close(got, want, F32_TOL, "float32")
+        close(replay(eng, {"b": toks}, [[("b", 45)]])["b"], want, F32_TOL, "whole")
+    else:
+        err = (got.double() - want).abs().amax(dim=1) / want.std()
+        assert err.median() < 0.08 and err.max() < 0.4, (err.median().item(), err.max().item())
+    eng.shutdown()
+
+
 def test_first_tokens_and_window_edges_in_prompts_and_decoding(tmp_path):
     """A window of 9 over prompts of 1, 2, 8, 9, 10 tokens and over decoded tokens that cross it one by one; key tiles of 64 crossed
     in the layers without a window; a portion that starts in the middle of a window."""
