@@ -43,8 +43,11 @@ typedef void* nvx_stream_t;
  *   4: direct-peer all-reduce (`nvx_peer_*`) and sharded sampling (`nvx_sample_shard`, `nvx_sample_pick`) added.
  *   8: layers with a 32-bit residual stream and per-sequence state (`nvx_boundary_norm`, `nvx_canon_conv`, `nvx_relu2`,
  *      `nvx_mingru_scan`) and latent attention (`nvx_latent_prep`, `nvx_latent_attn`) added.
- *   9: nvx_boundary_norm can apply the convolution of a decode step in the same launch. */
-#define NVX_ABI_VERSION 16
+ *   9: nvx_boundary_norm can apply the convolution of a decode step in the same launch.
+ *  17: several residual streams (`nvx_hyper_mix`), the real-gated recurrence (`nvx_rglru_scan`), a latent with a rotated key part
+ *      (`nvx_latent_rope_prep`), the softmax router with groups (`nvx_moe_route_softmax`), `nvx_short_conv`; nvx_softcap_attn gained a
+ *      sink and a gate per head. */
+#define NVX_ABI_VERSION 17
 
 /* Library identification and diagnostics. */
 int nvx_abi_version(void);
@@ -536,7 +539,9 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  *     (t - qo_indptr[b]) (and, with window > 0, only the last `window` of them: itself and the window - 1 before it):
  *     s_j = scale * q . k_j,  s_j <- cap tanh(s_j / cap) (cap > 0),  s_j <- s_j - r1[h] ln(1 + r2[h] (i - j)) (r1, r2 != null; i the
  *     query's position),  out = softmax(s) V; with vcs ((n_tok, vdim) float32: each query token's cos | sin, as nvx_attn_prep_store
- *     hands them out) the pairs of out are turned back by those angles (the counterpart of rotated values), with gate out is multiplied by sigmoid(gate[t]) (same layout as out).  Query head h reads
+ *     hands them out) the pairs of out are turned back by those angles (the counterpart of rotated values), with gate out is multiplied by
+ *     sigmoid(gate[t]) (same layout as out, or with gate_per_head one number per head: gate[t][h]).  With sink != 0 the softmax's sum
+ *     has one more term exp(sink_score) that carries no value: p_j = exp(s_j) / (exp(sink_score) + sum exp(s)).  Query head h reads
  *     key/value head h / (heads / kv_heads).  q (n_tok, heads * dim), k_cache (slots, kv_heads * dim), v_cache (slots, kv_heads *
  *     vdim), out (n_tok, heads * vdim).  n_split > 1 (for steps of few tokens): a (token, head)'s keys are dealt out over n_split
  *     workgroups whose partial results go to `part` (n_tok * heads * n_split * (vdim + 2) floats) and are merged by a second launch.
@@ -545,6 +550,9 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  *     keys in tiles of 32, weights as hi + lo 16-bit halves); scores and the softmax stay float32.
  * nvx_moe_route:  idx[t][k], wts[t][k] = the expert with the k-th largest logit of token t (ties: the lower id) and the sigmoid
  *     of that logit.
+ * nvx_moe_route_softmax:  scores = softmax(logits[t]) over all n_exp experts; with n_groups > 1 the experts form n_groups equal
+ *     groups of neighbours, a group counts as its largest score and only experts of the keep_groups best groups can be chosen; idx[t]
+ *     = the `top` largest scores among those (ties: the lower id), wts[t][k] = score / (sum of the chosen scores + norm_eps).
  * Expert e:  g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), y = g sigmoid(alpha g) (u + shift), result W_down y, with
  *     w_gu (experts, 2 ff, width) = rows [gate | up] and w_d (experts, width, ff).  (limit = infinity, alpha = 1, shift = 0: silu(g) u.)
  * nvx_moe_expert_rows:  out[t] = sum_k expert_idx[t][k](wts[t][k] * h[t]), or sum_k wts[t][k] * expert_idx[t][k](h[t]) if
@@ -562,6 +570,20 @@ int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv
  *     ws (n_seq * n_chunk_max * heads * dim * vdim floats; n_chunk_max >= the chunks of the longest portion); chunk 0: one walk.
  * nvx_postnorm_residual:  r = a y[t] (+ b y2[t]);  x[t] += r / rms(r) * w_post (w_post_n = 1: one number, = width: per channel);
  *     h_out[t] = x[t] / rms(x[t]) * w_next (w_next != null) or x[t] itself, in the format `fmt`.  rms(z) = sqrt(mean z^2 + eps).
+ * nvx_hyper_mix:  n_streams residual streams per token, x_out (n_tok, n_streams, width) float32.  With a result y (format `fmt`):
+ *     r = y[t] * scale (scale: width floats or null), and every stream at once from the old ones x_j' = sum_s mix[s * n_streams + j]
+ *     x_s + w_out[j] r; without: x_j' = x_j.  Old streams are read at x_in + t * in_tok_stride + s * in_stream_stride (stride 0: all
+ *     streams start from one row; x_in may be x_out).  Then u = sum_j w_in[j] x_j' (w_in null: the plain sum) and h_out[t] = u /
+ *     sqrt(mean u^2 + eps) * w_norm (h_out may be null).  At most 16 streams, width <= 15360.
+ * nvx_short_conv:  nvx_short_conv_silu with an optional bias per channel (added before the activation) and act 0 (none) or 1 (silu).
+ * nvx_rglru_scan:  per token and channel c of block b = c / block_width (j = c % block_width): r = sigmoid(gates[b][t][j] +
+ *     gate_bias[c]), i = sigmoid(gates[b][t][block_width + j] + gate_bias[width + c]) with gates (blocks, n_tok, 2 block_width) at the
+ *     given strides; a = exp(-rate[c] r); S <- a S + sqrt(1 - a^2) i u[t][c]; out[t][c] = S gelu_tanh(y[t][c]).  S (slots, width)
+ *     float32, zero at position 0; gates, sums and state float32.
+ * nvx_latent_rope_prep:  x[t] holds the queries at q_off (heads x [dim | rot]), [latent (kv_rank) | key part (rot)] at kv_off and one
+ *     gate pre-activation per head at g_off.  q_out[t] = the queries with their last `rot` entries per head turned in neighbouring
+ *     pairs by positions[t] * freq[i] (cos and sin times mag); cache[slots[t]] (row_len >= kv_rank + rot entries) = [latent / rms *
+ *     w_kv | key part turned the same way | zeros]; gate[t][h] = sigmoid(pre-activation), float32.
  * nvx_embed_scale:  x[t] = table[ids[t]] * scale (float32), h[t] the same in the table's format (h may be null).
  * nvx_tanh_cap:  out[i] = cap tanh(in[i] / cap) in float32 (cap <= 0: a copy).
  * nvx_skinny_proj:  out[t][n] = sum_k w[n][k] * f(x[t][k]) in float32, f = identity (in_act 0) or tanh (1); w float32 (n_out,
@@ -576,6 +598,20 @@ int nvx_head_norm_gate(const float* o, const float* w, int w_shared, const void*
 int nvx_short_conv_silu(const void* x, int64_t x_stride, int fmt, const float* w, int taps_n, float* state, int64_t n_slots,
                         const int32_t* tok_seq, const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot,
                         void* out, int64_t n_tok, int64_t n_seq, int64_t channels, nvx_stream_t stream);
+int nvx_short_conv(const void* x, int64_t x_stride, int fmt, const float* w, const float* bias, int act, int taps_n, float* state,
+                   int64_t n_slots, const int32_t* tok_seq, const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot,
+                   void* out, int64_t n_tok, int64_t n_seq, int64_t channels, nvx_stream_t stream);
+int nvx_rglru_scan(const void* y, int64_t y_stride, const void* u, int64_t u_stride, const void* gates, int64_t g_block_stride,
+                   int64_t g_tok_stride, int64_t block_width, const float* gate_bias, const float* rate, int fmt, float* state,
+                   int64_t n_slots, const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot, void* out,
+                   int64_t n_tok, int64_t n_seq, int64_t width, nvx_stream_t stream);
+int nvx_latent_rope_prep(const void* x, int64_t x_row_stride, int fmt, int64_t q_off, int64_t kv_off, int64_t g_off,
+                         const int64_t* positions, const double* freq, float mag, const float* w_kv, float eps,
+                         const int64_t* slots, void* q_out, void* cache, int64_t n_slots, int64_t row_len, float* gate,
+                         int64_t n_tok, int64_t heads, int64_t dim, int64_t rot, int64_t kv_rank, nvx_stream_t stream);
+int nvx_hyper_mix(const float* x_in, int64_t in_tok_stride, int64_t in_stream_stride, const void* y, int64_t y_stride, int fmt,
+                  const float* scale, const float* mix, const float* w_out, const float* w_in, const float* w_norm, float eps,
+                  float* x_out, void* h_out, int64_t n_tok, int64_t n_streams, int64_t width, nvx_stream_t stream);
 int nvx_token_shift_mix(const void* h, int64_t h_stride, int fmt, const float* mu, int n_mix, float* state, int64_t n_slots,
                         const int32_t* tok_seq, const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot,
                         void* out, int64_t n_tok, int64_t n_seq, int64_t width, nvx_stream_t stream);
@@ -601,7 +637,8 @@ int nvx_softcap_attn(const void* q, const void* k_cache, const void* v_cache, in
                      const int64_t* kv_start, const int32_t* kv_len, const int32_t* qo_indptr, const int32_t* tok_seq,
                      float scale, float cap, void* out, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
                      int n_split, float* part, int64_t window, const float* r1, const float* r2, const float* vcs,
-                     int v_interleaved, const void* gate, int64_t gate_stride, int64_t n_seq, int matrix_cores, nvx_stream_t stream);
+                     int v_interleaved, const void* gate, int64_t gate_stride, int gate_per_head, int sink, float sink_score,
+                     int64_t n_seq, int matrix_cores, nvx_stream_t stream);
 int nvx_softcap_attn_tile_fits(int fmt, int64_t dim, int64_t vdim, int turned_halves);
 int nvx_attn_prep_store(const void* x, int64_t x_stride, int fmt, int64_t q_off, int64_t k_off, int64_t v_off,
                         const int64_t* positions, const float* q_w, const float* k_w, int norm_mode, float eps, const double* freq,
@@ -619,6 +656,8 @@ int nvx_embed_scale(const int64_t* ids, const void* table, int fmt, int64_t voca
                     int64_t width, nvx_stream_t stream);
 int nvx_tanh_cap(const void* in, int fmt, float cap, float* out, int64_t n, nvx_stream_t stream);
 int nvx_moe_route(const float* logits, int64_t n_tok, int64_t n_exp, int64_t top, int32_t* idx, float* wts, nvx_stream_t stream);
+int nvx_moe_route_softmax(const float* logits, int64_t n_tok, int64_t n_exp, int64_t top, int64_t n_groups, int64_t keep_groups,
+                          float norm_eps, int32_t* idx, float* wts, nvx_stream_t stream);
 int64_t nvx_moe_expert_rows_max_width(int64_t ff);
 int nvx_moe_expert_rows(const void* h, int64_t h_stride, int fmt, const int32_t* idx, const float* wts, int64_t top,
                         const void* w_gu, const void* w_d, int64_t n_exp, float limit, float alpha, float shift, int weight_out,

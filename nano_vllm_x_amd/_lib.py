@@ -109,7 +109,8 @@ SIGNATURES = {
     "nvx_rope_vnorm_store": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_f32, _c_i32, _c_f32, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64,
                                       _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
     "nvx_softcap_attn": (_c_i32, [_c_vp, _c_vp, _c_vp, _c_i32, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64, _c_i64,
-                                  _c_i64, _c_i64, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_i32, _c_vp, _c_i64, _c_i64, _c_i32, _c_vp]),
+                                  _c_i64, _c_i64, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_i32, _c_vp, _c_i64, _c_i32, _c_i32, _c_f32, _c_i64,
+                                  _c_i32, _c_vp]),
     "nvx_softcap_attn_tile_fits": (_c_i32, [_c_i32, _c_i64, _c_i64, _c_i32]),
     "nvx_attn_prep_store": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_vp, _c_i32, _c_f32, _c_vp, _c_i32, _c_i32,
                                      _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp]),
@@ -128,6 +129,15 @@ SIGNATURES = {
     "nvx_moe_scatter_rows": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp]),
     "nvx_moe_glu": (_c_i32, [_c_vp, _c_i32, _c_f32, _c_f32, _c_f32, _c_vp, _c_i64, _c_i64, _c_vp]),
     "nvx_moe_gather_rows": (_c_i32, [_c_vp, _c_i32, _c_vp, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_vp]),
+    "nvx_short_conv": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_i32, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_i64,
+                                _c_i64, _c_i64, _c_vp]),
+    "nvx_rglru_scan": (_c_i32, [_c_vp, _c_i64, _c_vp, _c_i64, _c_vp, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_i32, _c_vp, _c_i64, _c_vp, _c_vp,
+                                _c_vp, _c_vp, _c_i64, _c_i64, _c_i64, _c_vp]),
+    "nvx_latent_rope_prep": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_i64, _c_i64, _c_i64, _c_vp, _c_vp, _c_f32, _c_vp, _c_f32, _c_vp, _c_vp, _c_vp,
+                                      _c_i64, _c_i64, _c_vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_vp]),
+    "nvx_hyper_mix": (_c_i32, [_c_vp, _c_i64, _c_i64, _c_vp, _c_i64, _c_i32, _c_vp, _c_vp, _c_vp, _c_vp, _c_vp, _c_f32, _c_vp, _c_vp, _c_i64,
+                               _c_i64, _c_i64, _c_vp]),
+    "nvx_moe_route_softmax": (_c_i32, [_c_vp, _c_i64, _c_i64, _c_i64, _c_i64, _c_i64, _c_f32, _c_vp, _c_vp, _c_vp]),
     "nvx_skinny_proj": (_c_i32, [_c_vp, _c_i64, _c_i32, _c_vp, _c_i32, _c_vp, _c_i64, _c_i64, _c_i64, _c_vp]),
 }
 

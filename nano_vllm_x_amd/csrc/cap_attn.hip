@@ -6,8 +6,9 @@
 //   - nvx_attn_prep_store: the same place for heads with a query/key RMS norm (per head, or over all heads of a row at once), a
 //     rotation in either pair layout, and values that are themselves rotated by their position before they are cached;
 //   - nvx_softcap_attn: the attention itself; scores, maxima, exponentials and sums are float32 in every format.  Optional: a
-//     sliding window, a logarithmic distance penalty per head, the read-out turned back by the query's position (the
-//     counterpart of rotated values) and multiplied by a sigmoid gate.
+//     sliding window, a logarithmic distance penalty per head, a sink (one more term in the softmax's sum, with a score of its
+//     own and no value), the read-out turned back by the query's position (the counterpart of rotated values) and multiplied by
+//     a sigmoid gate (one per element, or one per head).
 #include "fmt_dev.h"
 
 namespace NVX_NS {
@@ -160,10 +161,11 @@ __global__ __launch_bounds__(256) void attn_prep_store_kernel(const A* __restric
 // The end of an attention read-out for one (token, head): `so` holds its vdim values in LDS (every thread of the workgroup has
 // passed a barrier since they were written).  With `turn` (the query token's cos | sin row, vdim / 2 each, as nvx_attn_prep_store
 // hands it out) the pairs are turned BACK by those angles (values were cached turned by their own positions, so the weighted sum
-// is a sum of values in the query's frame); with a gate row every element is multiplied by sigmoid(gate).
+// is a sum of values in the query's frame); with a gate row every element is multiplied by sigmoid(gate): its own entry of the
+// row, or the row's one entry for the whole head (`gate_one`).
 template <typename A>
 __device__ __forceinline__ void attn_readout_end(float* so, int vdim, const float* __restrict__ turn, int interleaved,
-                                                 const A* __restrict__ gate_row, A* __restrict__ out_row, int n_threads) {
+                                                 const A* __restrict__ gate_row, bool gate_one, A* __restrict__ out_row, int n_threads) {
     if (turn) {
         const int vhalf = vdim / 2;
         for (int m = threadIdx.x; m < vhalf; m += n_threads) {
@@ -177,7 +179,7 @@ __device__ __forceinline__ void attn_readout_end(float* so, int vdim, const floa
     }
     for (int e = threadIdx.x; e < vdim; e += n_threads) {
         float v = so[e];
-        if (gate_row) v *= sigmoid_f(ld_f(gate_row, e));
+        if (gate_row) v *= sigmoid_f(ld_f(gate_row, gate_one ? 0 : e));
         st_f(out_row, e, v);
     }
 }
@@ -197,7 +199,8 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
                                                           int heads, int kv_heads, int dim, int vdim, int vec_v_ok, int n_split,
                                                           float* __restrict__ part, int window, const float* __restrict__ r1,
                                                           const float* __restrict__ r2, const float* __restrict__ vcs, int v_inter,
-                                                          const A* __restrict__ gate, int64_t gate_stride) {
+                                                          const A* __restrict__ gate, int64_t gate_stride, int gate_one, int sink,
+                                                          float sink_score) {
     extern __shared__ float sm[];
     float* sq = sm;                   // dim
     float* sacc = sq + dim;           // 4 * vdim
@@ -306,11 +309,13 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
     }
     if (lane == 0) { sml[wave] = m; sml[4 + wave] = l; }
     __syncthreads();
-    const float mm = fmaxf(fmaxf(sml[0], sml[1]), fmaxf(sml[2], sml[3]));
-    float f[4], total = 0.f;
+    float* pr = n_split > 1 ? part + ((t * heads + hd) * (int64_t)n_split + blockIdx.z) * (vdim + 2) : nullptr;
+    // a sink is one more term of the softmax's sum, with a score of its own and no value (a split's parts get it where they are merged)
+    const bool sunk = sink && !pr;
+    const float mm = fmaxf(fmaxf(fmaxf(sml[0], sml[1]), fmaxf(sml[2], sml[3])), sunk ? sink_score : -INFINITY);
+    float f[4], total = sunk ? expf(sink_score - mm) : 0.f;
 #pragma unroll
     for (int w = 0; w < 4; ++w) { f[w] = sml[w] == -INFINITY ? 0.f : expf(sml[w] - mm); total += sml[4 + w] * f[w]; }
-    float* pr = n_split > 1 ? part + ((t * heads + hd) * (int64_t)n_split + blockIdx.z) * (vdim + 2) : nullptr;
     for (int e = threadIdx.x; e < vdim; e += 256) {
         float o = 0.f;
 #pragma unroll
@@ -322,7 +327,8 @@ __global__ __launch_bounds__(256) void softcap_attn_kernel(const A* __restrict__
     if (pr && threadIdx.x == 0) { pr[0] = mm; pr[1] = total; }
     if (!pr && (vcs || gate)) {
         __syncthreads();
-        attn_readout_end<A>(sacc, vdim, vcs ? vcs + t * (int64_t)vdim : nullptr, v_inter, gate ? gate + t * gate_stride + (int64_t)hd * vdim : nullptr,
+        attn_readout_end<A>(sacc, vdim, vcs ? vcs + t * (int64_t)vdim : nullptr, v_inter,
+                            gate ? gate + t * gate_stride + (gate_one ? (int64_t)hd : (int64_t)hd * vdim) : nullptr, gate_one != 0,
                             out + t * (int64_t)heads * vdim + (int64_t)hd * vdim, 256);
     }
 }
@@ -367,7 +373,7 @@ __global__ __launch_bounds__(256) void softcap_attn_tile_kernel(const A* __restr
                                                                float scale, float cap, A* __restrict__ out, int heads, int kv_heads, int window,
                                                                const float* __restrict__ r1, const float* __restrict__ r2,
                                                                const float* __restrict__ vcs, int v_inter, const A* __restrict__ gate,
-                                                               int64_t gate_stride) {
+                                                               int64_t gate_stride, int gate_one, int sink, float sink_score) {
     constexpr int dim = DS * 32, vdim = VT * 16;
     __shared__ A vt_lds[vdim * VT_ROW];
     __shared__ int where[2];
@@ -539,6 +545,13 @@ __global__ __launch_bounds__(256) void softcap_attn_tile_kernel(const A* __restr
     l_run += xor16(l_run);
     l_run += xor32(l_run);
     if (!row_on) return;
+    if (sink) {                                                      // one more term of the sum, no value: the maximum may move to it
+        const float s2 = sink_score * LOG2E, m_new = fmaxf(m_run, s2);
+        const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+        l_run = l_run * alpha + __builtin_amdgcn_exp2f(s2 - m_new);
+#pragma unroll
+        for (int t = 0; t < VT; ++t) acc[t] *= alpha;
+    }
     const float inv = 1.0f / l_run;
 #pragma unroll
     for (int t = 0; t < VT; ++t) acc[t] *= inv;
@@ -569,10 +582,11 @@ __global__ __launch_bounds__(256) void softcap_attn_tile_kernel(const A* __restr
         }
     }
     A* orow = out + tok * heads * vdim + (int64_t)hd * vdim + 4 * g;
-    const A* grow = gate ? gate + tok * gate_stride + (int64_t)hd * vdim + 4 * g : nullptr;
+    const A* grow = gate && !gate_one ? gate + tok * gate_stride + (int64_t)hd * vdim + 4 * g : nullptr;
+    const float g_head = gate && gate_one ? sigmoid_f((float)gate[tok * gate_stride + hd]) : 1.0f;      // one gate for the whole head
 #pragma unroll
     for (int t = 0; t < VT; ++t) {
-        float o[4] = {acc[t][0], acc[t][1], acc[t][2], acc[t][3]};
+        float o[4] = {acc[t][0] * g_head, acc[t][1] * g_head, acc[t][2] * g_head, acc[t][3] * g_head};
         if (grow) {
             typedef A vec4 __attribute__((ext_vector_type(4)));
             const vec4 gv = *reinterpret_cast<const vec4*>(grow + t * 16);
@@ -587,13 +601,14 @@ __global__ __launch_bounds__(256) void softcap_attn_tile_kernel(const A* __restr
 template <typename A>
 __global__ __launch_bounds__(64) void softcap_merge_kernel(const float* __restrict__ part, int n_split, A* __restrict__ out, int vdim,
                                                           int heads, const float* __restrict__ vcs, int v_inter,
-                                                          const A* __restrict__ gate, int64_t gate_stride) {
+                                                          const A* __restrict__ gate, int64_t gate_stride, int gate_one, int sink,
+                                                          float sink_score) {
     __shared__ float so[512];
     const int64_t row = blockIdx.x;
     const float* pr = part + row * n_split * (vdim + 2);
-    float mm = -INFINITY;
+    float mm = sink ? sink_score : -INFINITY;
     for (int s = 0; s < n_split; ++s) mm = fmaxf(mm, pr[s * (vdim + 2)]);
-    float total = 0.f;
+    float total = sink ? expf(sink_score - mm) : 0.f;
     for (int s = 0; s < n_split; ++s) {
         const float m = pr[s * (vdim + 2)];
         total += m == -INFINITY ? 0.f : pr[s * (vdim + 2) + 1] * expf(m - mm);
@@ -610,7 +625,8 @@ __global__ __launch_bounds__(64) void softcap_merge_kernel(const float* __restri
     if (vcs || gate) {
         const int64_t t = row / heads;
         __syncthreads();
-        attn_readout_end<A>(so, vdim, vcs ? vcs + t * (int64_t)vdim : nullptr, v_inter, gate ? gate + t * gate_stride + (row % heads) * vdim : nullptr,
+        attn_readout_end<A>(so, vdim, vcs ? vcs + t * (int64_t)vdim : nullptr, v_inter,
+                            gate ? gate + t * gate_stride + (gate_one ? row % heads : (row % heads) * vdim) : nullptr, gate_one != 0,
                             out + row * vdim, 64);
     }
 }
@@ -677,8 +693,8 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
                                 const int64_t* kv_start, const int32_t* kv_len, const int32_t* qo_indptr, const int32_t* tok_seq,
                                 float scale, float cap, void* out, int64_t n_tok, int64_t heads, int64_t kv_heads, int64_t dim, int64_t vdim,
                                 int n_split, float* part, int64_t window, const float* r1, const float* r2, const float* vcs,
-                                int v_interleaved, const void* gate, int64_t gate_stride, int64_t n_seq, int matrix_cores,
-                                nvx_stream_t stream) {
+                                int v_interleaved, const void* gate, int64_t gate_stride, int gate_per_head, int sink, float sink_score,
+                                int64_t n_seq, int matrix_cores, nvx_stream_t stream) {
     NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_softcap_attn: fmt must be 0, 1 or 2");
     NVX_REQUIRE(n_tok >= 0 && n_tok <= 65535 && heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && dim <= 4096 && vdim > 0 && vdim <= 512,
                 NVX_EINVAL, "nvx_softcap_attn: bad sizes (at most 65535 tokens a step, key size <= 4096, value size <= 512)");
@@ -688,11 +704,11 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
     NVX_REQUIRE((r1 != nullptr) == (r2 != nullptr), NVX_EINVAL, "nvx_softcap_attn: the distance penalty takes both of its numbers per head");
     NVX_REQUIRE(window >= 0 && window < (1ll << 31), NVX_EINVAL, "nvx_softcap_attn: bad window");
     NVX_REQUIRE(!vcs || (vdim % 2 == 0 && nvx_aligned16(vcs)), NVX_EINVAL, "nvx_softcap_attn: a read-out that is turned back has an even size");
-    NVX_REQUIRE(!gate || gate_stride >= heads * vdim, NVX_EINVAL, "nvx_softcap_attn: row stride of the gate");
+    NVX_REQUIRE(!gate || gate_stride >= (gate_per_head ? heads : heads * vdim), NVX_EINVAL, "nvx_softcap_attn: row stride of the gate");
     // steps of many tokens in a 16-bit format, sizes the tile kernel is built for, 8-byte rows of the gate: the matrix cores
     if (matrix_cores && nvx_softcap_attn_tile_fits(fmt, dim, vdim, vcs != nullptr && !v_interleaved) && qo_indptr && n_split == 1 && n_seq > 0 &&
         nvx_aligned16(q) && nvx_aligned16(k_cache) && nvx_aligned16(v_cache) && (reinterpret_cast<uintptr_t>(out) & 7u) == 0 &&
-        (!gate || ((reinterpret_cast<uintptr_t>(gate) & 7u) == 0 && gate_stride % 4 == 0))) {
+        (!gate || gate_per_head || ((reinterpret_cast<uintptr_t>(gate) & 7u) == 0 && gate_stride % 4 == 0))) {
         NVX_REQUIRE((n_tok + TILE_Q - 1) / TILE_Q + n_seq <= 65535, NVX_EINVAL, "nvx_softcap_attn: too many tokens or sequences in one step");
         const dim3 tgrid((unsigned)heads, (unsigned)((n_tok + TILE_Q - 1) / TILE_Q + n_seq));
 #define NVX_TILE_ATTN(DS, VT)                                                                                                            \
@@ -700,7 +716,8 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
                                          (const typename tile_fmt<A_>::type*)q, (const typename tile_fmt<A_>::type*)k_cache,            \
                                          (const typename tile_fmt<A_>::type*)v_cache, kv_indices, kv_start, kv_len, qo_indptr, (int)n_seq, scale, \
                                          cap, (typename tile_fmt<A_>::type*)out, (int)heads, (int)kv_heads, (int)window, r1, r2, vcs,    \
-                                         v_interleaved, (const typename tile_fmt<A_>::type*)gate, gate_stride))
+                                         v_interleaved, (const typename tile_fmt<A_>::type*)gate, gate_stride, gate_per_head, sink,   \
+                                         sink_score))
 #define NVX_TILE_ATTN_V(DS)                                                       \
     do {                                                                          \
         if (vdim == 64) NVX_TILE_ATTN(DS, 4);                                     \
@@ -722,7 +739,7 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
                                          (const A_*)q, (const A_*)k_cache, (const A_*)v_cache, kv_indices, kv_start, kv_len, qo_indptr,      \
                                          tok_seq, scale, cap, (A_*)out, (int)heads, (int)kv_heads, (int)dim, (int)vdim,       \
                                          (int)nvx_aligned16(v_cache), n_split, part, (int)window, r1, r2, vcs, v_interleaved,   \
-                                         (const A_*)gate, gate_stride))
+                                         (const A_*)gate, gate_stride, gate_per_head, sink, sink_score))
 #define NVX_CAP_ATTN(EPL) do { if (vec) NVX_CAP_ATTN_V(EPL, true); else NVX_CAP_ATTN_V(EPL, false); } while (0)
     const bool vec = fmt != 2 && dim % 8 == 0 && nvx_aligned16(k_cache);
     if (vdim <= 64) NVX_CAP_ATTN(1);
@@ -733,7 +750,7 @@ extern "C" int nvx_softcap_attn(const void* q, const void* k_cache, const void* 
     if (n_split > 1)
         NVX_FMT_CALL(fmt, hipLaunchKernelGGL(softcap_merge_kernel<A_>, dim3((unsigned)(n_tok * heads)), dim3(64), 0, (hipStream_t)stream,
                                              (const float*)part, n_split, (A_*)out, (int)vdim, (int)heads, vcs, v_interleaved, (const A_*)gate,
-                                             gate_stride));
+                                             gate_stride, gate_per_head, sink, sink_score));
 #undef NVX_CAP_ATTN
     return nvx_check_launch("nvx_softcap_attn");
 }

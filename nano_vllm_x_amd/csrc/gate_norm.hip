@@ -102,6 +102,56 @@ __global__ __launch_bounds__(256) void postnorm_residual_kernel(const A* __restr
     }
 }
 
+// Several residual streams per token (x: (tokens, streams, width) float32) and the sublayer boundary between them.  Per token t:
+//   with a result y:   r = y[t] * scale (scale: one number per channel, or none);
+//                      every stream at once from the old ones:  x_j' = sum_s mix[s][j] x_s + w_out[j] r      (mix indexed [from][to])
+//   without one:       x_j' = x_j  (x_in may be ONE row per token that all streams start from: in_stream_stride 0)
+//   then what the next sublayer reads:  u = sum_j w_in[j] x_j'  (w_in null: the plain sum),  h[t] = u / rms(u) * w_norm.
+// A thread holds the old values of its columns for all streams before it writes any, so x_in may be x_out.  u waits in LDS for
+// the row's mean square.
+template <typename A, int MAXS>
+__global__ __launch_bounds__(256) void hyper_mix_kernel(const float* x_in, int64_t in_tok_stride, int64_t in_stream_stride,
+                                                       const A* __restrict__ y, int64_t y_stride, const float* __restrict__ scale,
+                                                       const float* __restrict__ mix, const float* __restrict__ w_out,
+                                                       const float* __restrict__ w_in, const float* __restrict__ w_norm, float eps,
+                                                       float* x_out, A* __restrict__ h_out, int n_streams, int width) {
+    extern __shared__ float su[];                 // width
+    __shared__ float s_mix[MAXS * MAXS], s_out[MAXS], s_in[MAXS], red[4];
+    const int64_t t = blockIdx.x;
+    for (int i = threadIdx.x; i < n_streams * n_streams; i += 256) s_mix[(i / n_streams) * MAXS + (i % n_streams)] = mix ? mix[i] : 0.f;
+    for (int i = threadIdx.x; i < n_streams; i += 256) { s_out[i] = w_out ? w_out[i] : 0.f; s_in[i] = w_in ? w_in[i] : 1.0f; }
+    __syncthreads();
+    const float* xr = x_in + t * in_tok_stride;
+    float* xo = x_out + t * (int64_t)n_streams * width;
+    const A* yr = y ? y + t * y_stride : nullptr;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < width; c += 256) {
+        float old[MAXS];
+#pragma unroll
+        for (int s = 0; s < MAXS; ++s) old[s] = s < n_streams ? xr[s * in_stream_stride + c] : 0.f;
+        const float r = yr ? ld_f(yr, c) * (scale ? scale[c] : 1.0f) : 0.f;
+        float u = 0.f;
+#pragma unroll
+        for (int j = 0; j < MAXS; ++j) {
+            if (j < n_streams) {
+                float v = old[j];
+                if (yr) {
+                    v = s_out[j] * r;
+#pragma unroll
+                    for (int s = 0; s < MAXS; ++s) if (s < n_streams) v += s_mix[s * MAXS + j] * old[s];
+                }
+                if (yr || x_out != x_in || in_stream_stride == 0) xo[(int64_t)j * width + c] = v;
+                u += s_in[j] * v;
+            }
+        }
+        su[c] = u;
+        ss += u * u;
+    }
+    if (!h_out) return;
+    const float rn = 1.0f / sqrtf(block256_sum(ss, red) / (float)width + eps);
+    for (int c = threadIdx.x; c < width; c += 256) st_f(h_out, t * (int64_t)width + c, su[c] * rn * (w_norm ? w_norm[c] : 1.0f));
+}
+
 // x[t] = table[ids[t]] * scale (float32), h[t] = the same in the activations' format
 template <typename A>
 __global__ __launch_bounds__(256) void embed_scale_kernel(const int64_t* __restrict__ ids, const A* __restrict__ table, int64_t vocab, float scale,
@@ -284,6 +334,32 @@ extern "C" int nvx_postnorm_residual(const void* y, int64_t y_stride, const void
                                          y_stride, (const A_*)y2, y2_stride, a, b, w_post, (int)w_post_n, x, w_next, (int)w_next_n, eps, (A_*)h_out,
                                          (int)width));
     return nvx_check_launch("nvx_postnorm_residual");
+}
+
+extern "C" int nvx_hyper_mix(const float* x_in, int64_t in_tok_stride, int64_t in_stream_stride, const void* y, int64_t y_stride, int fmt,
+                             const float* scale, const float* mix, const float* w_out, const float* w_in, const float* w_norm, float eps,
+                             float* x_out, void* h_out, int64_t n_tok, int64_t n_streams, int64_t width, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_hyper_mix: fmt must be 0, 1 or 2");
+    NVX_REQUIRE(n_tok >= 0 && n_streams >= 1 && n_streams <= 16 && width > 0, NVX_EINVAL, "nvx_hyper_mix: bad sizes (at most 16 streams)");
+    NVX_REQUIRE(width <= 15360, NVX_EUNSUPPORTED, "nvx_hyper_mix: a row must fit LDS as float32 (width <= 15360)");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(x_in && x_out, NVX_EINVAL, "nvx_hyper_mix: null pointer");
+    NVX_REQUIRE(in_tok_stride >= width && (in_stream_stride == 0 || in_stream_stride >= width), NVX_EINVAL, "nvx_hyper_mix: strides of the streams");
+    NVX_REQUIRE(!y || (y_stride >= width && mix && w_out), NVX_EINVAL, "nvx_hyper_mix: a result needs the mixing matrix and its output weights");
+    NVX_REQUIRE(x_in != x_out || (in_tok_stride == n_streams * width && in_stream_stride == width), NVX_EINVAL,
+                "nvx_hyper_mix: streams updated in place keep their layout");
+    const size_t lds = (size_t)width * sizeof(float);
+#define NVX_HYPER(MAXS)                                                                                                               \
+    NVX_FMT_CALL(fmt, hipLaunchKernelGGL((hyper_mix_kernel<A_, MAXS>), dim3((unsigned)n_tok), dim3(256), lds, (hipStream_t)stream, x_in, \
+                                         in_tok_stride, in_stream_stride, (const A_*)y, y_stride, scale, mix, w_out, w_in, w_norm, eps, \
+                                         x_out, (A_*)h_out, (int)n_streams, (int)width))
+    if (n_streams <= 1) NVX_HYPER(1);
+    else if (n_streams <= 2) NVX_HYPER(2);
+    else if (n_streams <= 4) NVX_HYPER(4);
+    else if (n_streams <= 8) NVX_HYPER(8);
+    else NVX_HYPER(16);
+#undef NVX_HYPER
+    return nvx_check_launch("nvx_hyper_mix");
 }
 
 extern "C" int nvx_embed_scale(const int64_t* ids, const void* table, int fmt, int64_t vocab, float scale, float* x, void* h, int64_t n_tok,

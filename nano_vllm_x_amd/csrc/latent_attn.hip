@@ -46,6 +46,64 @@ __global__ __launch_bounds__(256) void latent_prep_kernel(
         gate[t * heads + h] = 1.0f / (1.0f + expf(-la_ld(r, q_rank + kv_rank + h)));
 }
 
+// ---- the same place for a latent with a rotated key part ---------------------------------------------------------------------
+// x[t] holds, at their offsets: the queries (heads x [dim plain | rot rotated]), the down projection [latent (kv_rank) | one rotated
+// key part (rot) that all heads share], one output-gate pre-activation per head.
+//   q_out[t]        = the queries, their rotated parts turned by the token's position
+//   cache[slot[t]]  = [ latent / rms * w_kv | key part turned by the position | zeros up to row_len ]
+//   gate[t][h]      = sigmoid(pre-activation)                      (float32)
+// Pairs are neighbours (2i, 2i + 1); the angle position * freq[i] is formed and brought into [-pi, pi] in double precision (freq:
+// float64, rot / 2), cosine and sine are float32 and multiplied by `mag`.  The cache row is a key row for the folded queries
+// [W_uk^T q_plain | q_rotated] and its latent part the value row, so the attention over latents serves this layout as it is.
+template <typename A>
+__global__ __launch_bounds__(256) void latent_rope_prep_kernel(
+    const A* __restrict__ x, int64_t x_stride, int q_off, int kv_off, int g_off, const int64_t* __restrict__ positions,
+    const double* __restrict__ freq, float mag, const float* __restrict__ w_kv, float eps, const int64_t* __restrict__ slots,
+    A* __restrict__ q_out, A* __restrict__ cache, int64_t n_slots, int row_len, float* __restrict__ gate, int heads, int dim, int rot,
+    int kv_rank) {
+    extern __shared__ float cs[];                // rot: cos | sin
+    __shared__ float red[4];
+    const int64_t t = blockIdx.x;
+    const A* r = x + t * x_stride;
+    const int half = rot / 2;
+    const double pos = (double)positions[t];
+    for (int i = threadIdx.x; i < half; i += 256) {
+        const double two_pi = 6.283185307179586476925286766559;
+        const double a = pos * freq[i];
+        float sn, c;
+        sincosf((float)(a - two_pi * rint(a / two_pi)), &sn, &c);
+        cs[i] = c * mag;
+        cs[half + i] = sn * mag;
+    }
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < kv_rank; c += 256) { const float v = la_ld(r, kv_off + c); ss += v * v; }
+    const float rk = 1.0f / sqrtf(la_block_sum(ss, red) / (float)kv_rank + eps);        // (its barriers also publish cs)
+    const int hd = dim + rot;
+    for (int i = threadIdx.x; i < heads * hd; i += 256) {
+        const int d = i % hd - dim;
+        float v = la_ld(r, q_off + i);
+        if (d >= 0) {
+            const int m = d >> 1;
+            v = (d & 1) ? v * cs[m] + la_ld(r, q_off + i - 1) * cs[half + m] : v * cs[m] - la_ld(r, q_off + i + 1) * cs[half + m];
+        }
+        la_st(q_out, t * (int64_t)heads * hd + i, v);
+    }
+    for (int h = threadIdx.x; h < heads; h += 256) gate[t * heads + h] = 1.0f / (1.0f + expf(-la_ld(r, g_off + h)));
+    const int64_t slot = slots[t];
+    if (slot < 0 || slot >= n_slots) return;
+    A* row = cache + slot * row_len;
+    for (int c = threadIdx.x; c < row_len; c += 256) {
+        float v = 0.f;
+        if (c < kv_rank) v = la_ld(r, kv_off + c) * rk * w_kv[c];
+        else if (c < kv_rank + rot) {
+            const int d = c - kv_rank, m = d >> 1;
+            const float own = la_ld(r, kv_off + c);
+            v = (d & 1) ? own * cs[m] + la_ld(r, kv_off + c - 1) * cs[half + m] : own * cs[m] - la_ld(r, kv_off + c + 1) * cs[half + m];
+        }
+        la_st(row, c, v);
+    }
+}
+
 // ---- attention over the cached latents ------------------------------------------------------------------------------
 // One workgroup per (query token, group of HG heads).  Keys come in tiles of 256: first every thread scores one key
 // against the group's folded queries (held in LDS), the tile's weights go to LDS, then every thread owns output
@@ -571,6 +629,25 @@ extern "C" int nvx_latent_prep(const void* x, int64_t x_row_stride, int fmt, con
     NVX_FMT_DISPATCH(fmt, launch_prep<A_>(x, x_row_stride, w_q, w_kv, eps, slots, cq, cache, n_slots, gate, n_tok, (int)q_rank, (int)kv_rank,
                                           (int)heads, (hipStream_t)stream));
     return nvx_check_launch("nvx_latent_prep");
+}
+
+extern "C" int nvx_latent_rope_prep(const void* x, int64_t x_row_stride, int fmt, int64_t q_off, int64_t kv_off, int64_t g_off,
+                                    const int64_t* positions, const double* freq, float mag, const float* w_kv, float eps,
+                                    const int64_t* slots, void* q_out, void* cache, int64_t n_slots, int64_t row_len, float* gate,
+                                    int64_t n_tok, int64_t heads, int64_t dim, int64_t rot, int64_t kv_rank, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_latent_rope_prep: fmt must be 0, 1 or 2");
+    NVX_REQUIRE(n_tok >= 0 && heads > 0 && dim >= 0 && rot >= 0 && rot % 2 == 0 && rot <= 8192 && dim + rot > 0 && kv_rank > 0 && n_slots >= 0 &&
+                    row_len >= kv_rank + rot && heads * (dim + rot) < (1 << 30) && row_len < (1 << 30),
+                NVX_EINVAL, "nvx_latent_rope_prep: bad sizes (the rotated part is even, a cache row holds the latent and the rotated key part)");
+    NVX_REQUIRE(q_off >= 0 && kv_off >= 0 && g_off >= 0 && x_row_stride >= q_off + heads * (dim + rot) && x_row_stride >= kv_off + kv_rank + rot &&
+                    x_row_stride >= g_off + heads, NVX_EINVAL, "nvx_latent_rope_prep: a part lies outside a row");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(x && positions && (freq || rot == 0) && w_kv && slots && q_out && cache && gate, NVX_EINVAL, "nvx_latent_rope_prep: null pointer");
+    NVX_FMT_DISPATCH(fmt, hipLaunchKernelGGL(latent_rope_prep_kernel<A_>, dim3((unsigned)n_tok), dim3(256), (size_t)(rot + 2) * sizeof(float),
+                                             (hipStream_t)stream, (const A_*)x, x_row_stride, (int)q_off, (int)kv_off, (int)g_off, positions, freq,
+                                             mag, w_kv, eps, slots, (A_*)q_out, (A_*)cache, n_slots, (int)row_len, gate, (int)heads, (int)dim,
+                                             (int)rot, (int)kv_rank));
+    return nvx_check_launch("nvx_latent_rope_prep");
 }
 
 extern "C" int nvx_latent_attn(const void* q, const void* cache, int fmt, const int32_t* kv_indices, const int64_t* kv_start,

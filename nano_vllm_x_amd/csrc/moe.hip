@@ -1,6 +1,7 @@
 // Mixture of small gated feed-forward experts; a choice's weight scales the chosen expert's INPUT (sigmoid routers) or its
 // OUTPUT (weight_out: fixed weights from a table).
 //   - nvx_moe_route: the `top` largest router logits of every token -> expert ids and sigmoid scores (float32);
+//   - nvx_moe_route_softmax: softmax scores, experts in groups of which only the best may be chosen, weights renormalised;
 //   - nvx_moe_expert_rows: a token's experts evaluated row by row of their weights: the form for steps of few tokens, where
 //     every chosen expert's weights have to be streamed once per token anyway;
 //   - nvx_moe_order / nvx_moe_scatter_rows / nvx_moe_glu / nvx_moe_gather_rows: the pieces around per-expert matrix products
@@ -28,6 +29,55 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
         idx[t * top + k] = best;
         wts[t * top + k] = sigmoid_f(bz);
     }
+}
+
+// Softmax router with groups: scores = softmax(logits) over all experts; the experts form n_groups equal groups of neighbours, a
+// group counts as its best score, and only experts of the keep_groups best groups can be chosen (n_groups <= 1: all of them);
+// the `top` largest scores among those are chosen (ties: the lower id) and their scores, divided by their sum + norm_eps, are the
+// weights.  One thread per token; everything float32.
+__global__ __launch_bounds__(256) void moe_route_softmax_kernel(const float* __restrict__ logits, int n_exp, int top, int n_groups,
+                                                               int keep_groups, float norm_eps, int32_t* __restrict__ idx,
+                                                               float* __restrict__ wts, int64_t n_tok) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= n_tok) return;
+    const float* z = logits + t * n_exp;
+    float zmax = -INFINITY;
+    for (int e = 0; e < n_exp; ++e) zmax = fmaxf(zmax, z[e]);
+    float denom = 0.f;
+    for (int e = 0; e < n_exp; ++e) denom += expf(z[e] - zmax);
+    // the groups that stay: keep_groups times the best group not yet taken (a group's score is its largest logit: the softmax keeps the order)
+    uint64_t kept[4] = {0, 0, 0, 0};                       // n_groups <= 256
+    const bool grouped = n_groups > 1 && keep_groups < n_groups;
+    const int per = grouped ? n_exp / n_groups : n_exp;
+    if (grouped) {
+        for (int k = 0; k < keep_groups; ++k) {
+            int best = -1;
+            float bz = -INFINITY;
+            for (int g = 0; g < n_groups; ++g) {
+                if ((kept[g >> 6] >> (g & 63)) & 1) continue;
+                float gm = -INFINITY;
+                for (int e = g * per; e < (g + 1) * per; ++e) gm = fmaxf(gm, z[e]);
+                if (best < 0 || gm > bz) { best = g; bz = gm; }
+            }
+            kept[best >> 6] |= 1ull << (best & 63);
+        }
+    }
+    float sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+        int best = -1;
+        float bz = -INFINITY;
+        for (int e = 0; e < n_exp; ++e) {
+            if (grouped) { const int g = e / per; if (!((kept[g >> 6] >> (g & 63)) & 1)) continue; }
+            bool taken = false;
+            for (int j = 0; j < k; ++j) taken |= idx[t * top + j] == e;
+            if (!taken && (best < 0 || z[e] > bz)) { best = e; bz = z[e]; }
+        }
+        idx[t * top + k] = best;
+        const float sc = expf(bz - zmax) / denom;
+        wts[t * top + k] = sc;
+        sum += sc;
+    }
+    for (int k = 0; k < top; ++k) wts[t * top + k] /= (sum + norm_eps);
 }
 
 __device__ __forceinline__ float glu_act(float g, float u, float limit, float alpha, float shift) {
@@ -257,6 +307,19 @@ extern "C" int nvx_moe_route(const float* logits, int64_t n_tok, int64_t n_exp, 
     hipLaunchKernelGGL(moe_route_kernel, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, (hipStream_t)stream, logits, (int)n_exp, (int)top,
                        idx, wts, n_tok);
     return nvx_check_launch("nvx_moe_route");
+}
+
+extern "C" int nvx_moe_route_softmax(const float* logits, int64_t n_tok, int64_t n_exp, int64_t top, int64_t n_groups, int64_t keep_groups,
+                                     float norm_eps, int32_t* idx, float* wts, nvx_stream_t stream) {
+    NVX_REQUIRE(n_tok >= 0 && n_exp > 0 && n_exp < (1 << 20) && top > 0 && top <= n_exp, NVX_EINVAL, "nvx_moe_route_softmax: bad sizes");
+    NVX_REQUIRE(n_groups >= 0 && n_groups <= 256 && (n_groups <= 1 || (n_exp % n_groups == 0 && keep_groups >= 1 && keep_groups <= n_groups &&
+                                                                      keep_groups * (n_exp / n_groups) >= top)),
+                NVX_EINVAL, "nvx_moe_route_softmax: groups must divide the experts (at most 256 groups) and the kept groups must hold `top` experts");
+    if (n_tok == 0) return NVX_OK;
+    NVX_REQUIRE(logits && idx && wts, NVX_EINVAL, "nvx_moe_route_softmax: null pointer");
+    hipLaunchKernelGGL(moe_route_softmax_kernel, dim3((unsigned)((n_tok + 255) / 256)), dim3(256), 0, (hipStream_t)stream, logits, (int)n_exp,
+                       (int)top, (int)n_groups, (int)keep_groups, norm_eps, idx, wts, n_tok);
+    return nvx_check_launch("nvx_moe_route_softmax");
 }
 
 extern "C" int64_t nvx_moe_expert_rows_max_width(int64_t ff) {

@@ -368,6 +368,125 @@ __global__ __launch_bounds__(256) void mingru_step_kernel(
     }
 }
 
+// ---- real-gated linear recurrent unit ----------------------------------------------------------------------------------
+// Per token and channel c (block b = c / block_width, j = c % block_width), all of it float32:
+//   r = sigmoid(gates[b][t][j] + gate_bias[c]),  i = sigmoid(gates[b][t][block_width + j] + gate_bias[width + c])
+//   log a = -rate[c] * r,  a = exp(log a),  S <- a S + sqrt(1 - a^2) * i * u[t][c],  out = S * gelu_tanh(y[t][c])
+// `gates` is what a batched product over the blocks leaves: (blocks, tokens, 2 * block_width), recurrence gate | input gate;
+// `rate` is the channel's constant (the design's multiplier times softplus of its parameter).  1 - a^2 is formed as
+// -expm1(2 log a), which keeps its leading digits where a is close to one.  The scan is the one of the minGRU kernel:
+// S_t = a_t S_(t-1) + b_t by segments of the time axis that are chained through LDS.
+struct RglruIn {
+    const void* y; int64_t y_stride;
+    const void* u; int64_t u_stride;
+    const void* gates; int64_t g_block_stride, g_tok_stride;
+    const float* gate_bias; const float* rate;
+    int block_width, width;
+};
+
+__device__ __forceinline__ float gelu_tanh_f(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+}
+
+// (a, b, output gate) of token row `t` (a row of the step) and channel c
+template <typename A>
+__device__ __forceinline__ void rglru_cell(const RglruIn& in, int64_t t, int c, float& a, float& b, float& g) {
+    const int blk = c / in.block_width, j = c - blk * in.block_width;
+    const A* gr = (const A*)in.gates + blk * in.g_block_stride + t * in.g_tok_stride;
+    const float r = sigm<A>(ldf(gr, j) + in.gate_bias[c]);
+    const float i = sigm<A>(ldf(gr, in.block_width + j) + in.gate_bias[in.width + c]);
+    const float log_a = -in.rate[c] * r;
+    a = expf(log_a);
+    b = sqrtf(fmaxf(-expm1f(2.0f * log_a), 0.f)) * i * ldf((const A*)in.u, t * in.u_stride + c);
+    g = gelu_tanh_f(ldf((const A*)in.y, t * in.y_stride + c));
+}
+
+template <typename A, int SEG>
+__global__ __launch_bounds__(256) void rglru_scan_kernel(RglruIn in, float* __restrict__ state, const int32_t* __restrict__ qo_indptr,
+                                                        const int64_t* __restrict__ pos0, const int32_t* __restrict__ state_slot,
+                                                        A* __restrict__ out) {
+    __shared__ float agg_a[GRU_NSEG][GRU_CB], agg_b[GRU_NSEG][GRU_CB];
+    const int b = blockIdx.y;
+    const int slot = state_slot[b];
+    if (slot < 0) return;
+    const int64_t q0 = qo_indptr[b];
+    const int64_t n = qo_indptr[b + 1] - q0;
+    if (n <= 0) return;
+    const int width = in.width;
+    const int seg = threadIdx.x >> 4, cl = (threadIdx.x & 15) * 2;
+    const int c = blockIdx.x * GRU_CB + cl;
+    const bool live[2] = {c < width, c + 1 < width};
+    const bool had = pos0[b] > 0;
+    float carry[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k) carry[k] = (live[k] && had) ? state[(int64_t)slot * width + c + k] : 0.f;
+    for (int64_t base = 0; base < n; base += SEG * GRU_NSEG) {
+        const int64_t t0 = base + (int64_t)seg * SEG;
+        float pa[2][SEG], ps[2][SEG], gg[2][SEG];
+        float ar[2] = {1.f, 1.f}, sr[2] = {0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < SEG; ++i) {
+            const int64_t t = t0 + i;
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                gg[k][i] = 0.f;
+                if (t < n && live[k]) {
+                    float a, bb, g;
+                    rglru_cell<A>(in, q0 + t, c + k, a, bb, g);
+                    sr[k] = a * sr[k] + bb;
+                    ar[k] *= a;
+                    gg[k][i] = g;
+                }
+                pa[k][i] = ar[k];
+                ps[k][i] = sr[k];
+            }
+        }
+        __syncthreads();                   // the previous round's readers are done
+#pragma unroll
+        for (int k = 0; k < 2; ++k) { agg_a[seg][cl + k] = ar[k]; agg_b[seg][cl + k] = sr[k]; }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+            float in_s = carry[k];         // state before this thread's first token
+            for (int q = 0; q < seg; ++q) in_s = agg_a[q][cl + k] * in_s + agg_b[q][cl + k];
+            float last = in_s;
+            for (int q = seg; q < GRU_NSEG; ++q) last = agg_a[q][cl + k] * last + agg_b[q][cl + k];
+            carry[k] = last;               // state after the round's last token (segments past the end are identities)
+            if (live[k]) {
+#pragma unroll
+                for (int i = 0; i < SEG; ++i) {
+                    const int64_t t = t0 + i;
+                    if (t < n) stf(out, (q0 + t) * (int64_t)width + c + k, (pa[k][i] * in_s + ps[k][i]) * gg[k][i]);
+                }
+            }
+        }
+    }
+    if (seg == 0) {
+#pragma unroll
+        for (int k = 0; k < 2; ++k) if (live[k]) state[(int64_t)slot * width + c + k] = carry[k];
+    }
+}
+
+// one token per sequence (a decode step): thread = (sequence, channel)
+template <typename A>
+__global__ __launch_bounds__(256) void rglru_step_kernel(RglruIn in, float* __restrict__ state, const int64_t* __restrict__ pos0,
+                                                        const int32_t* __restrict__ state_slot, A* __restrict__ out, int64_t n_seq) {
+    const int width = in.width;
+    const int64_t total = n_seq * (int64_t)width;
+    for (int64_t id = (int64_t)blockIdx.x * 256 + threadIdx.x; id < total; id += (int64_t)gridDim.x * 256) {
+        const int64_t b = id / width;
+        const int c = (int)(id - b * width);
+        const int slot = state_slot[b];
+        if (slot < 0) { stf(out, id, 0.f); continue; }
+        float a, bb, g;
+        rglru_cell<A>(in, b, c, a, bb, g);
+        float* sp = state + (int64_t)slot * width + c;
+        const float s = a * (pos0[b] > 0 ? *sp : 0.f) + bb;
+        *sp = s;
+        stf(out, id, s * g);
+    }
+}
+
 template <typename A>
 static int launch_boundary(const void* m, int64_t m_stride, const float* res, const float* w_post, float* hist, int64_t hist_stride,
                            int hist_slot, int n_mix, const float* mix, float* x_out, const float* w_pre, float* y_f32, void* y_act,
@@ -422,6 +541,19 @@ static void launch_mingru(const void* zxg, int64_t row_stride, float* state, con
     }
     hipLaunchKernelGGL((mingru_scan_kernel<A, 8>), dim3((unsigned)((width + GRU_CB - 1) / GRU_CB), (unsigned)n_seq), dim3(256), 0, s, (const A*)zxg,
                        row_stride, state, qo_indptr, pos0, state_slot, (A*)out, width);
+}
+
+template <typename A>
+static void launch_rglru(const RglruIn& in, float* state, const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot, void* out,
+                         int64_t n_seq, hipStream_t s) {
+    if (!qo_indptr) {
+        int64_t blocks = (n_seq * in.width + 255) / 256;
+        if (blocks > 256 * 64) blocks = 256 * 64;
+        hipLaunchKernelGGL(rglru_step_kernel<A>, dim3((unsigned)blocks), dim3(256), 0, s, in, state, pos0, state_slot, (A*)out, n_seq);
+        return;
+    }
+    hipLaunchKernelGGL((rglru_scan_kernel<A, 8>), dim3((unsigned)((in.width + GRU_CB - 1) / GRU_CB), (unsigned)n_seq), dim3(256), 0, s, in, state,
+                       qo_indptr, pos0, state_slot, (A*)out);
 }
 
 }  // namespace NVX_NS
@@ -496,4 +628,20 @@ extern "C" int nvx_mingru_scan(const void* zxg, int64_t row_stride, int fmt, flo
     NVX_REQUIRE(qo_indptr || n_tok == n_seq, NVX_EINVAL, "nvx_mingru_scan: without qo_indptr every sequence has one token");
     NVX_FMT_DISPATCH(fmt, launch_mingru<A_>(zxg, row_stride, state, qo_indptr, pos0, state_slot, out, n_seq, (int)width, (hipStream_t)stream));
     return nvx_check_launch("nvx_mingru_scan");
+}
+
+extern "C" int nvx_rglru_scan(const void* y, int64_t y_stride, const void* u, int64_t u_stride, const void* gates, int64_t g_block_stride,
+                              int64_t g_tok_stride, int64_t block_width, const float* gate_bias, const float* rate, int fmt, float* state,
+                              int64_t n_slots, const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot, void* out,
+                              int64_t n_tok, int64_t n_seq, int64_t width, nvx_stream_t stream) {
+    NVX_REQUIRE(fmt >= 0 && fmt <= 2, NVX_EINVAL, "nvx_rglru_scan: fmt must be 0, 1 or 2");
+    NVX_REQUIRE(n_tok >= 0 && n_seq >= 0 && n_seq <= 65535 && width > 0 && width < (1 << 30) && n_slots >= 0 && block_width > 0 &&
+                    width % block_width == 0 && y_stride >= width && u_stride >= width && g_tok_stride >= 2 * block_width && g_block_stride >= 0,
+                NVX_EINVAL, "nvx_rglru_scan: bad sizes");
+    if (n_tok == 0 || n_seq == 0) return NVX_OK;
+    NVX_REQUIRE(y && u && gates && gate_bias && rate && state && pos0 && state_slot && out, NVX_EINVAL, "nvx_rglru_scan: null pointer");
+    NVX_REQUIRE(qo_indptr || n_tok == n_seq, NVX_EINVAL, "nvx_rglru_scan: without qo_indptr every sequence has one token");
+    const RglruIn in = {y, y_stride, u, u_stride, gates, g_block_stride, g_tok_stride, gate_bias, rate, (int)block_width, (int)width};
+    NVX_FMT_DISPATCH(fmt, launch_rglru<A_>(in, state, qo_indptr, pos0, state_slot, out, n_seq, (hipStream_t)stream));
+    return nvx_check_launch("nvx_rglru_scan");
 }

@@ -1,5 +1,5 @@
 // Token mixers that carry a matrix per head from token to token, and the small steps in front of them:
-//   - short causal convolution over time per channel followed by silu, its last inputs kept per sequence;
+//   - short causal convolution over time per channel (optional bias, optional silu), its last inputs kept per sequence;
 //   - token shift: every token's row mixed with its predecessor's by per-channel weights, the last row kept per sequence;
 //   - three recurrences over a (key size x value size) memory per head:
 //       mlstm   exponential input gate and sigmoid forget gate stabilised by a running maximum, normaliser vector;
@@ -16,12 +16,13 @@
 
 namespace NVX_NS {
 
-// ---- short convolution + silu --------------------------------------------------------------------------------------------
-// out[t][c] = silu(sum_j w[j][c] * in[t - (taps_n - 1) + j][c]) over the tokens of t's own sequence; inputs before this step
-// come from state[slot] (taps_n - 1 rows, oldest first), inputs before the sequence's start are zero.
+// ---- short convolution (+ bias, + silu) ------------------------------------------------------------------------------------
+// out[t][c] = act(bias[c] + sum_j w[j][c] * in[t - (taps_n - 1) + j][c]) over the tokens of t's own sequence (bias may be null; act 0:
+// none, 1: silu); inputs before this step come from state[slot] (taps_n - 1 rows, oldest first), inputs before the sequence's
+// start are zero.
 template <typename A>
-__global__ __launch_bounds__(256) void short_conv_silu_kernel(const A* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
-                                                             int taps_n, const float* __restrict__ state, const int32_t* __restrict__ tok_seq,
+__global__ __launch_bounds__(256) void short_conv_kernel(const A* __restrict__ x, int64_t x_stride, const float* __restrict__ w,
+                                                        const float* __restrict__ bias, int act, int taps_n, const float* __restrict__ state, const int32_t* __restrict__ tok_seq,
                                                              const int32_t* __restrict__ qo_indptr, const int64_t* __restrict__ pos0,
                                                              const int32_t* __restrict__ state_slot, A* __restrict__ out, int channels) {
     const int64_t t = blockIdx.y;
@@ -31,7 +32,7 @@ __global__ __launch_bounds__(256) void short_conv_silu_kernel(const A* __restric
     const int hist_n = taps_n - 1;
     const bool has_state = s.pos0 > 0 && s.slot >= 0;
     for (int c = blockIdx.x * 256 + threadIdx.x; c < channels; c += gridDim.x * 256) {
-        float acc = 0.f;
+        float acc = bias ? bias[c] : 0.f;
         for (int i = 0; i < taps_n; ++i) {
             const int64_t src = j - (hist_n - i);
             float v = 0.f;
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(256) void short_conv_silu_kernel(const A* __restric
             else if (has_state) v = state[((int64_t)s.slot * hist_n + (hist_n + src)) * channels + c];
             acc += w[(int64_t)i * channels + c] * v;
         }
-        st_f(out, t * (int64_t)channels + c, acc * sigmoid_f(acc));
+        st_f(out, t * (int64_t)channels + c, act == 1 ? acc * sigmoid_f(acc) : acc);
     }
 }
 
@@ -503,23 +504,30 @@ using namespace NVX_NS;
     NVX_REQUIRE(pos0 && state_slot, NVX_EINVAL, name ": null layout");                                                              \
     NVX_REQUIRE(qo_indptr || n_tok == n_seq, NVX_EINVAL, name ": without qo_indptr every sequence has one token")
 
-extern "C" int nvx_short_conv_silu(const void* x, int64_t x_stride, int fmt, const float* w, int taps_n, float* state, int64_t n_slots,
-                                   const int32_t* tok_seq, const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot,
-                                   void* out, int64_t n_tok, int64_t n_seq, int64_t channels, nvx_stream_t stream) {
-    NVX_LAYOUT_OK("nvx_short_conv_silu");
-    NVX_REQUIRE(channels > 0 && channels < (1 << 30) && x_stride >= channels && taps_n >= 1 && taps_n <= 64 && n_slots >= 0 && n_tok <= 65535,
-                NVX_EINVAL, "nvx_short_conv_silu: bad sizes");
-    NVX_REQUIRE(x && w && out && (state || taps_n == 1), NVX_EINVAL, "nvx_short_conv_silu: null pointer");
-    NVX_REQUIRE((tok_seq != nullptr) == (qo_indptr != nullptr), NVX_EINVAL, "nvx_short_conv_silu: tok_seq and qo_indptr go together");
+extern "C" int nvx_short_conv(const void* x, int64_t x_stride, int fmt, const float* w, const float* bias, int act, int taps_n, float* state,
+                              int64_t n_slots, const int32_t* tok_seq, const int32_t* qo_indptr, const int64_t* pos0,
+                              const int32_t* state_slot, void* out, int64_t n_tok, int64_t n_seq, int64_t channels, nvx_stream_t stream) {
+    NVX_LAYOUT_OK("nvx_short_conv");
+    NVX_REQUIRE(channels > 0 && channels < (1 << 30) && x_stride >= channels && taps_n >= 1 && taps_n <= 64 && n_slots >= 0 && n_tok <= 65535 &&
+                    (act == 0 || act == 1), NVX_EINVAL, "nvx_short_conv: bad sizes, or an activation other than 0 (none) and 1 (silu)");
+    NVX_REQUIRE(x && w && out && (state || taps_n == 1), NVX_EINVAL, "nvx_short_conv: null pointer");
+    NVX_REQUIRE((tok_seq != nullptr) == (qo_indptr != nullptr), NVX_EINVAL, "nvx_short_conv: tok_seq and qo_indptr go together");
     const unsigned cx = (unsigned)((channels + 255) / 256);
     NVX_FMT_CALL(fmt, {
-        hipLaunchKernelGGL(short_conv_silu_kernel<A_>, dim3(cx, (unsigned)n_tok), dim3(256), 0, (hipStream_t)stream, (const A_*)x, x_stride, w,
-                           taps_n, (const float*)state, tok_seq, qo_indptr, pos0, state_slot, (A_*)out, (int)channels);
+        hipLaunchKernelGGL(short_conv_kernel<A_>, dim3(cx, (unsigned)n_tok), dim3(256), 0, (hipStream_t)stream, (const A_*)x, x_stride, w, bias,
+                           act, taps_n, (const float*)state, tok_seq, qo_indptr, pos0, state_slot, (A_*)out, (int)channels);
         if (taps_n > 1)
             hipLaunchKernelGGL(tail_rows_kernel<A_>, dim3(cx, (unsigned)n_seq), dim3(256), 0, (hipStream_t)stream, (const A_*)x, x_stride,
                                taps_n - 1, state, qo_indptr, pos0, state_slot, (int)channels);
     });
-    return nvx_check_launch("nvx_short_conv_silu");
+    return nvx_check_launch("nvx_short_conv");
+}
+
+extern "C" int nvx_short_conv_silu(const void* x, int64_t x_stride, int fmt, const float* w, int taps_n, float* state, int64_t n_slots,
+                                   const int32_t* tok_seq, const int32_t* qo_indptr, const int64_t* pos0, const int32_t* state_slot,
+                                   void* out, int64_t n_tok, int64_t n_seq, int64_t channels, nvx_stream_t stream) {
+    return nvx_short_conv(x, x_stride, fmt, w, nullptr, 1, taps_n, state, n_slots, tok_seq, qo_indptr, pos0, state_slot, out, n_tok, n_seq,
+                          channels, stream);
 }
 
 extern "C" int nvx_token_shift_mix(const void* h, int64_t h_stride, int fmt, const float* mu, int n_mix, float* state, int64_t n_slots,

@@ -1,5 +1,6 @@
-"""Mixtures of small gated feed-forward experts: behind a sigmoid router whose score scales an expert's input, or chosen by a
-table of token ids with fixed weights on the experts' outputs."""
+"""Mixtures of small gated feed-forward experts: behind a sigmoid router whose score scales an expert's input, behind a softmax
+router with groups whose renormalised scores weigh the experts' outputs, or chosen by a table of token ids with fixed weights on
+the experts' outputs."""
 from __future__ import annotations
 
 import torch
@@ -123,3 +124,24 @@ class TableMoE(ExpertBank):
             idx, wts = self.choices(input_ids)
             return self.run(h, idx, wts, decode_step, weight_out=True)
         return self.run(h, plan["idx"], plan["wts"], decode_step, weight_out=True, order=plan["order"])
+
+
+class GroupedSoftmaxMoE(ExpertBank):
+    """scores = softmax(W_router h) over all experts (float32).  The experts form `groups` equal groups of neighbours; a group counts
+    as its best score and only experts of the `keep` best groups can be chosen (groups None or 1: no such limit).  Every token takes
+    the `top` largest scores among those, the weights are these scores divided by their sum + norm_eps, and they weigh the experts'
+    OUTPUTS.  Expert: g = min(W_gate x, limit), u = clamp(W_up x, -limit, limit), W_down (g * sigmoid(alpha * g) * (u + shift))."""
+
+    def __init__(self, width: int, experts: int, top: int, ff: int, limit: float, alpha: float, shift: float = 1.0, groups=None, keep=None,
+                 norm_eps: float = 1e-20):
+        super().__init__(width, experts, top, ff, limit, alpha, shift)
+        self.groups, self.keep = int(groups or 0), int(keep or 0)
+        if self.groups > 1:
+            if experts % self.groups or not 1 <= self.keep <= self.groups or self.keep * (experts // self.groups) < top:
+                raise ValueError("groups must divide the experts and the kept groups must hold `top` experts")
+        self.norm_eps = float(norm_eps)
+        self.router = nn.Parameter(torch.zeros(experts, width, dtype=torch.float32))
+
+    def forward(self, h: torch.Tensor, decode_step: bool = False) -> torch.Tensor:
+        idx, wts = ops.moe_route_softmax(ops.skinny_proj(h, self.router), self.top, self.groups, self.keep, self.norm_eps)
+        return self.run(h, idx, wts, decode_step, weight_out=True)

@@ -167,3 +167,47 @@ class DecayLinearAttention(nn.Module):
 
     def forward(self, h: torch.Tensor, md) -> torch.Tensor:
         return self.mix(self.in_proj(h), 0, md)
+
+
+class RGLRU(nn.Module):
+    """Recurrent block around a real-gated linear recurrent unit (S. De, S. L. Smith et al., "Griffin: Mixing Gated Linear
+    Recurrences with Local Attention for Efficient Language Models").  Two branches of `inner` channels: y = gelu_tanh(W_y h + b_y),
+    and u = causal convolution per channel (taps, with a bias, no activation) of W_x h + b_x.  The channels form `blocks` equal
+    blocks; within block b the gates are r = sigmoid(A_b u_b + a_b), i = sigmoid(B_b u_b + b_b) with square matrices A_b, B_b.  Then
+    a = exp(-decay_scale * r * softplus(lam)), S <- a S + sqrt(1 - a^2) * i * u (from S = 0, the first token like every other), and
+    the layer returns W_o (S * y).  State: S (float32) and the convolution's last taps - 1 inputs.
+    The two branch projections are one matrix product, the two gate maps of all blocks one batched product; gates, decay and state are
+    float32 inside the scan kernel; the channel's constant decay_scale * softplus(lam) is formed once, when the weights are in place."""
+
+    def __init__(self, width: int, inner: int, blocks: int, taps: int, decay_scale: float, state_name):
+        super().__init__()
+        if inner % blocks:
+            raise ValueError("the channels must divide into the blocks")
+        self.width, self.inner, self.blocks, self.taps, self.decay_scale, self.state_name = width, inner, blocks, taps, float(decay_scale), state_name
+        bw = inner // blocks
+        self.in_proj = nn.Linear(width, 2 * inner, bias=True)              # rows: y | x
+        self.conv_w = _f32(taps, inner)                                    # row j: the tap taps - 1 - j tokens back
+        self.conv_b = _f32(inner)
+        self.gate_w = nn.Parameter(torch.empty(blocks, bw, 2 * bw))        # per block: input channel -> recurrence gate | input gate
+        self.gate_b = _f32(2, inner)                                       # rows: recurrence gate | input gate
+        self.lam = _f32(inner)
+        self.register_buffer("rate", torch.zeros(inner, dtype=torch.float32), persistent=False)
+        self.o_proj = nn.Linear(inner, width, bias=False)
+
+    def finalize(self):
+        """After the weights are loaded: the constant factor of every channel's decay exponent."""
+        self.rate.copy_(self.decay_scale * F.softplus(self.lam.detach().double()).float())
+
+    def state_shapes(self) -> dict:
+        shapes = {(self.state_name, "S"): (self.inner,)}
+        if self.taps > 1:
+            shapes[(self.state_name, "conv")] = (self.taps - 1, self.inner)
+        return shapes
+
+    def forward(self, h: torch.Tensor, md) -> torch.Tensor:
+        n, t = self.state_name, h.shape[0]
+        yx = self.in_proj(h)
+        u = ops.short_conv(yx[:, self.inner:], self.conv_w, md.cache.state((n, "conv")) if self.taps > 1 else None, md.layout, bias=self.conv_b)
+        gates = torch.bmm(u.view(t, self.blocks, -1).transpose(0, 1), self.gate_w)      # (blocks, T, 2 * block width)
+        s = ops.rglru_scan(yx[:, :self.inner], u, gates, self.gate_b, self.rate, md.cache.state((n, "S")), md.layout)
+        return self.o_proj(s)

@@ -42,12 +42,16 @@ class RotaryEmbedding(nn.Module):
 
 
 def rotary_frequencies(dims: int, base: float, scaling: dict | None = None):
-    """(frequencies, magnitude) of a rotation of `dims` dimensions in pairs (i, i + dims / 2): f_i = base^(-2i / dims), float64
-    (dims / 2).  `scaling` = {factor, original, fast, slow} stretches the slow pairs (YaRN: B. Peng, J. Quesnelle, H. Fan,
-    E. Shippole, "YaRN: Efficient Context Window Extension of Large Language Models"): a pair that completes `turns`
-    turns over `original` positions has index d(turns) = dims ln(original / (2 pi turns)) / (2 ln base); between lo =
-    floor(d(fast)) and hi = ceil(d(slow)) (clipped to the table) a ramp goes from 0 to 1, a frequency becomes f / factor
-    where the ramp is 1 and stays f where it is 0, and cos and sin are multiplied by 0.1 ln(factor) + 1."""
+    """(frequencies, magnitude) of a rotation of `dims` dimensions in dims / 2 pairs: f_i = base^(-2i / dims), float64 (dims / 2).
+    `scaling` stretches the slow pairs, in one of two ways that its keys tell apart.
+    {factor, original, fast, slow} (YaRN: B. Peng, J. Quesnelle, H. Fan, E. Shippole, "YaRN: Efficient Context Window Extension of
+    Large Language Models"): a pair that completes `turns` turns over `original` positions has index d(turns) = dims ln(original /
+    (2 pi turns)) / (2 ln base); between lo = floor(d(fast)) and hi = ceil(d(slow)) (clipped to the table) a ramp goes from 0 to 1,
+    a frequency becomes f / factor where the ramp is 1 and stays f where it is 0, and cos and sin are multiplied by
+    0.1 ln(factor) + 1.
+    {factor, original, low, high} (bands of wavelength, as the Llama 3.1 models scale theirs): with wavelength L = 2 pi / f, f stays
+    where L < original / high, becomes f / factor where L > original / low, and between the two is the blend (1 - s) f / factor + s f
+    with s = (original / L - low) / (high - low); the magnitude stays 1."""
     import math
 
     idx = torch.arange(dims // 2, dtype=torch.float64)
@@ -55,6 +59,13 @@ def rotary_frequencies(dims: int, base: float, scaling: dict | None = None):
     if not scaling:
         return freq, 1.0
     factor, original = float(scaling["factor"]), float(scaling["original"])
+    if "low" in scaling or "high" in scaling:
+        low, high = float(scaling["low"]), float(scaling["high"])
+        wave = 2.0 * math.pi / freq
+        s = ((original / wave - low) / (high - low)) if high != low else torch.zeros_like(freq)
+        blend = (1.0 - s) * freq / factor + s * freq
+        out = torch.where(wave < original / high, freq, torch.where(wave > original / low, freq / factor, blend))
+        return out, 1.0
 
     def index_of(turns: float) -> float:
         return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(float(base)))

@@ -1061,14 +1061,15 @@ SOFTCAP_SPLITS = 4
 
 def softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, layout: StepLayout, scale: float, cap: float, heads: int,
                  kv_heads: int, dim: int, vdim: int, n_split: Optional[int] = None, window: int = 0, r1=None, r2=None, v_turn=None,
-                 v_interleaved: bool = False, gate=None, matrix_cores: bool = True):
+                 v_interleaved: bool = False, gate=None, matrix_cores: bool = True, sink_score: Optional[float] = None):
     """Causal attention of q (T, heads * dim) over cached rows: sequence b's tokens are at slots kv_indices[kv_start[b] :
     kv_start[b] + kv_len[b]]; scores scale * q . k pass cap * tanh(. / cap) (cap <= 0: not) before the softmax.
     `window` > 0: a token sees itself and the window - 1 tokens before it.  `r1`, `r2` (heads, float32): r1 ln(1 + r2 (i - j)) is
     taken off the score of key j for the query at position i.  `v_turn` (T, vdim) float32, every query token's cos | sin as
     attn_prep_store returns them: the read-out's pairs ((m, m + vdim / 2), or (2m, 2m + 1) if `v_interleaved`) are turned back by
     those angles, undoing the turn attn_prep_store gave the values.  `gate`
-    (T, heads * vdim): the read-out times sigmoid(gate).  Steps of many tokens in a 16-bit format, with key and value sizes of 64,
+    (T, heads * vdim), or (T, heads) with one number per head: the read-out times sigmoid(gate).  `sink_score`: the softmax's sum has
+    one more term exp(sink_score) that carries no value (0.0: one is added to the denominator).  Steps of many tokens in a 16-bit format, with key and value sizes of 64,
     96 or 128, run on the matrix cores unless `matrix_cores` is False.  Returns (T, heads * vdim) in q's format."""
     _dev(q, k_cache, v_cache, kv_indices, kv_start, kv_len, r1, r2, v_turn, gate)
     _need((r1 is None) == (r2 is None), "softcap_attn: r1 and r2 go together")
@@ -1078,7 +1079,9 @@ def softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, layout: Step
             _need(a.numel() == heads, "softcap_attn: r1 and r2 have one number per head")
     _need(v_turn is None or (v_turn.dtype == F32 and v_turn.is_contiguous() and v_turn.shape == (q.shape[0], vdim) and vdim % 2 == 0),
           "softcap_attn: v_turn must be float32 (T, vdim)")
-    _need(gate is None or (gate.shape == (q.shape[0], heads * vdim) and gate.stride(1) == 1 and gate.dtype == q.dtype), "softcap_attn: gate shape / format")
+    _need(gate is None or (gate.dim() == 2 and gate.shape[0] == q.shape[0] and gate.shape[1] in (heads, heads * vdim) and gate.stride(1) == 1 and
+                           gate.dtype == q.dtype), "softcap_attn: gate shape / format")
+    gate_per_head = gate is not None and gate.shape[1] == heads and vdim != 1
     t = q.shape[0]
     _need(q.shape == (t, heads * dim) and q.is_contiguous() and t == layout.n_tok, "softcap_attn: q must be contiguous (T, heads * dim)")
     n_slots = k_cache.shape[0]
@@ -1097,7 +1100,8 @@ def softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, layout: Step
     _lib.check(lib.nvx_softcap_attn(_ptr(q), _ptr(k_cache), _ptr(v_cache), _fmt(q), _ptr(kv_indices), _ptr(kv_start), _ptr(kv_len),
                                     _ptr(layout.qo_indptr), _ptr(layout.tok_seq), float(scale), float(cap), _ptr(out), t, heads, kv_heads, dim,
                                     vdim, n_split, _ptr(part), int(window or 0), _ptr(r1), _ptr(r2), _ptr(v_turn), int(bool(v_interleaved)),
-                                    _ptr(gate), gate.stride(0) if gate is not None else 0, layout.n_seq, int(bool(matrix_cores)), _stream()),
+                                    _ptr(gate), gate.stride(0) if gate is not None else 0, int(gate_per_head), int(sink_score is not None),
+                                    float(sink_score or 0.0), layout.n_seq, int(bool(matrix_cores)), _stream()),
                "nvx_softcap_attn")
     return out
 
@@ -1344,3 +1348,131 @@ def skinny_proj(x, w, in_act: str = "none"):
     _lib.check(lib.nvx_skinny_proj(_ptr(x), x.stride(0), _fmt(x), _ptr(w), {"none": 0, "tanh": 1}[in_act], _ptr(out), x.shape[0], w.shape[0],
                                    x.shape[1], _stream()), "nvx_skinny_proj")
     return out
+
+
+# ---------------------------------------------------------------------------------------------
+# several residual streams, the real-gated recurrence, a latent with a rotated key part, the softmax router with groups
+# ---------------------------------------------------------------------------------------------
+def hyper_mix(x, y=None, scale=None, mix=None, w_out=None, w_in=None, w_norm=None, eps: float = 0.0, n_streams: Optional[int] = None,
+              out_dtype=None, want_h: bool = True):
+    """Residual streams x (T, streams, width) float32 and a sublayer boundary.  With a result y (T, width): r = y * scale (scale:
+    (width) or None) and every stream at once from the old ones, x_j <- sum_s mix[s, j] x_s + w_out[j] r (in place).  x may also be
+    (T, width) with `n_streams`: the one row every stream starts from; the streams are then made.  Returns (x, h) with h = u /
+    rms(u) * w_norm for u = sum_j w_in[j] x_j (w_in None: the plain sum; w_norm None: ones), in `out_dtype` (default: y's)."""
+    _dev(x, y, scale, mix, w_out, w_in, w_norm)
+    _f32c(x, "hyper_mix: x")
+    if x.dim() == 2:
+        _need(n_streams is not None and n_streams >= 1 and y is None, "hyper_mix: one row per token starts n_streams streams, and has no result yet")
+        t, width = x.shape
+        x_out = torch.empty((t, n_streams, width), dtype=F32, device=x.device)
+        tok_stride, stream_stride = width, 0
+    else:
+        _need(x.dim() == 3, "hyper_mix: x must be (T, streams, width)")
+        t, n_streams, width = x.shape
+        x_out, tok_stride, stream_stride = x, n_streams * width, width
+    if y is not None:
+        _need(y.shape == (t, width) and y.stride(1) == 1, "hyper_mix: y must be (T, width) with unit inner stride")
+        _need(mix is not None and w_out is not None, "hyper_mix: a result needs the mixing matrix and its output weights")
+    for name, a, n in (("scale", scale, width), ("mix", mix, n_streams * n_streams), ("w_out", w_out, n_streams), ("w_in", w_in, n_streams),
+                       ("w_norm", w_norm, width)):
+        if a is not None:
+            _f32c(a, "hyper_mix: " + name)
+            _need(a.numel() == n, f"hyper_mix: {name} size")
+    dtype = out_dtype or (y.dtype if y is not None else None)
+    _need(not want_h or dtype in _FMT, "hyper_mix: output format")
+    _need(y is None or dtype is None or y.dtype == dtype, "hyper_mix: y and the output share one format")
+    h = torch.empty((t, width), dtype=dtype, device=x.device) if want_h else None
+    fmt = _FMT[dtype] if dtype is not None else _fmt(y)
+    lib = _lib.load()
+    _lib.check(lib.nvx_hyper_mix(_ptr(x), tok_stride, stream_stride, _ptr(y), y.stride(0) if y is not None else 0, fmt, _ptr(scale), _ptr(mix),
+                                 _ptr(w_out), _ptr(w_in), _ptr(w_norm), float(eps), _ptr(x_out), _ptr(h), t, n_streams, width, _stream()),
+               "nvx_hyper_mix")
+    return x_out, h
+
+
+def short_conv(x, w, state, layout: StepLayout, bias=None, act: str = "none"):
+    """act(bias + causal convolution over time per channel): short_conv_silu with an optional bias (channels, float32) and `act`
+    "none" or "silu".  x (T, channels) (rows may be a slice of wider rows); w (taps, channels) float32, row j multiplying the input
+    taps - 1 - j tokens back; state (slots, taps - 1, channels) float32.  Returns (T, channels) in x's format."""
+    _dev(x, w, state, bias)
+    _need(x.dim() == 2 and x.stride(1) == 1, "short_conv: x must be (T, channels) with unit inner stride")
+    t, ch = x.shape
+    _f32c(w, "short_conv: w")
+    taps = w.shape[0]
+    _need(w.dim() == 2 and w.shape[1] == ch and t == layout.n_tok, "short_conv: shapes")
+    if bias is not None:
+        _f32c(bias, "short_conv: bias")
+        _need(bias.numel() == ch, "short_conv: bias size")
+    n_slots = 0
+    if taps > 1:
+        _f32c(state, "short_conv: state")
+        _need(state.dim() == 3 and state.shape[1:] == (taps - 1, ch), "short_conv: state shape")
+        n_slots = state.shape[0]
+    out = torch.empty((t, ch), dtype=x.dtype, device=x.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_short_conv(_ptr(x), x.stride(0), _fmt(x), _ptr(w), _ptr(bias), {"none": 0, "silu": 1}[act], taps,
+                                  _ptr(state) if taps > 1 else None, n_slots, _ptr(layout.tok_seq), *_layout_args(layout), _ptr(out), t,
+                                  layout.n_seq, ch, _stream()), "nvx_short_conv")
+    return out
+
+
+def rglru_scan(y, u, gates, gate_bias, rate, state, layout: StepLayout):
+    """Real-gated linear recurrence over each sequence's tokens.  y, u (T, width) (rows may be slices of wider rows): the gelu
+    branch's pre-activation and the recurrence's input; gates (blocks, T, 2 * block_width): recurrence-gate | input-gate
+    pre-activations of every block of channels; gate_bias (2, width), rate (width) float32; state (slots, width) float32, continued
+    and written back.  a = exp(-rate * sigmoid(r)), S <- a S + sqrt(1 - a^2) sigmoid(i) u.  Returns S * gelu_tanh(y), (T, width)."""
+    _dev(y, u, gates, gate_bias, rate, state)
+    t, width = u.shape
+    _need(y.shape == (t, width) and y.stride(1) == 1 and u.stride(1) == 1 and y.dtype == u.dtype == gates.dtype, "rglru_scan: y, u (T, width) in one format")
+    _need(gates.dim() == 3 and gates.shape[1] == t and gates.stride(2) == 1 and gates.shape[2] % 2 == 0 and gates.shape[0] * gates.shape[2] == 2 * width,
+          "rglru_scan: gates must be (blocks, T, 2 * width / blocks)")
+    for a, what, n in ((gate_bias, "gate_bias", 2 * width), (rate, "rate", width)):
+        _f32c(a, "rglru_scan: " + what)
+        _need(a.numel() == n, f"rglru_scan: {what} size")
+    _f32c(state, "rglru_scan: state")
+    _need(t == layout.n_tok and state.dim() == 2 and state.shape[1] == width, "rglru_scan: shapes")
+    out = torch.empty((t, width), dtype=u.dtype, device=u.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_rglru_scan(_ptr(y), y.stride(0), _ptr(u), u.stride(0), _ptr(gates), gates.stride(0), gates.stride(1), gates.shape[2] // 2,
+                                  _ptr(gate_bias), _ptr(rate), _fmt(u), _ptr(state), state.shape[0], *_layout_args(layout), _ptr(out), t,
+                                  layout.n_seq, width, _stream()), "nvx_rglru_scan")
+    return out
+
+
+def latent_rope_prep(x, offsets, positions, freq, mag: float, w_kv, eps: float, slots, cache, heads: int, dim: int, rot: int):
+    """After the fused projection x (T, columns) holding, at the three column `offsets`, the queries (heads x [dim | rot]), the down
+    projection [latent (kv_rank) | key part (rot)] and one gate pre-activation per head.  The last `rot` entries of every query head
+    and the key part are turned in neighbouring pairs by positions * freq (float64, rot / 2; cos and sin times `mag`); the latent is
+    RMS-normed with w_kv (kv_rank, float32); cache[slots[t]] = [latent | key part | zeros] (cache: (slots, row) with row >= kv_rank +
+    rot).  Returns (queries (T, heads * (dim + rot)), gate (T, heads) float32 = sigmoid)."""
+    _dev(x, positions, freq, w_kv, slots, cache)
+    _need(x.dim() == 2 and x.stride(1) == 1, "latent_rope_prep: x must be (T, columns) with unit inner stride")
+    t = x.shape[0]
+    _f32c(w_kv, "latent_rope_prep: w_kv")
+    kv_rank = w_kv.numel()
+    _need(positions.dtype == torch.int64 and positions.is_contiguous() and positions.numel() == t, "latent_rope_prep: positions must be int64 (T)")
+    _need(slots.dtype == torch.int64 and slots.is_contiguous() and slots.numel() == t, "latent_rope_prep: slots must be int64 (T)")
+    _need(rot == 0 or (freq.dtype == torch.float64 and freq.is_contiguous() and freq.numel() == rot // 2), "latent_rope_prep: freq must be float64 (rot / 2)")
+    _need(cache.dtype == x.dtype and cache.is_contiguous() and cache.dim() == 2 and cache.shape[1] >= kv_rank + rot, "latent_rope_prep: cache")
+    q = torch.empty((t, heads * (dim + rot)), dtype=x.dtype, device=x.device)
+    gate = torch.empty((t, heads), dtype=F32, device=x.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_latent_rope_prep(_ptr(x), x.stride(0), _fmt(x), offsets[0], offsets[1], offsets[2], _ptr(positions), _ptr(freq) if rot else None,
+                                        float(mag), _ptr(w_kv), float(eps), _ptr(slots), _ptr(q), _ptr(cache), cache.shape[0], cache.shape[1],
+                                        _ptr(gate), t, heads, dim, rot, kv_rank, _stream()), "nvx_latent_rope_prep")
+    return q, gate
+
+
+def moe_route_softmax(logits, top: int, n_groups: int = 0, keep_groups: int = 0, norm_eps: float = 0.0):
+    """logits (T, experts) float32 -> (ids (T, top) int32, weights (T, top) float32).  Scores are the softmax over all experts; with
+    n_groups > 1 the experts form equal groups of neighbours, a group counts as its best score, and only experts of the keep_groups
+    best groups can be chosen; the `top` largest scores are taken (ties: the lower id) and divided by their sum + norm_eps."""
+    _dev(logits)
+    _f32c(logits, "moe_route_softmax: logits")
+    t, n_exp = logits.shape
+    idx = torch.empty((t, top), dtype=torch.int32, device=logits.device)
+    wts = torch.empty((t, top), dtype=F32, device=logits.device)
+    lib = _lib.load()
+    _lib.check(lib.nvx_moe_route_softmax(_ptr(logits), t, n_exp, top, int(n_groups or 0), int(keep_groups or 0), float(norm_eps), _ptr(idx),
+                                         _ptr(wts), _stream()), "nvx_moe_route_softmax")
+    return idx, wts

@@ -29,8 +29,13 @@ def _gibavik():
     return GibavikConfig.from_dict, GibavikForCausalLM
 
 
+def _ladusun():
+    from .ladusun import LadusunConfig, LadusunForCausalLM
+    return LadusunConfig.from_dict, LadusunForCausalLM
+
+
 # architecture name (config.json "architectures"[0] or "architecture") -> loader of (config reader, model class)
-ARCHITECTURES = {"Qwen3ForCausalLM": _qwen3, "Kabidra": _kabidra, "Meronex": _meronex, "Gibavik": _gibavik}
+ARCHITECTURES = {"Qwen3ForCausalLM": _qwen3, "Kabidra": _kabidra, "Meronex": _meronex, "Gibavik": _gibavik, "Ladusun": _ladusun}
 
 
 def architecture_of(config: dict) -> str:

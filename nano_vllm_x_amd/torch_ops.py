@@ -84,7 +84,8 @@ _DEFS = {
                         "Tensor(b!) v_cache, int heads, int kv_heads, int dim, int vdim) -> Tensor",
     "softcap_attn": "(Tensor q, Tensor k_cache, Tensor v_cache, Tensor kv_indices, Tensor kv_start, Tensor kv_len, Tensor pos0, "
                     "Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq, float scale, float cap, int heads, int kv_heads, int dim, int vdim, "
-                    "int window=0, Tensor? r1=None, Tensor? r2=None, Tensor? v_turn=None, bool v_interleaved=False, Tensor? gate=None) -> Tensor",
+                    "int window=0, Tensor? r1=None, Tensor? r2=None, Tensor? v_turn=None, bool v_interleaved=False, Tensor? gate=None, "
+                    "float? sink_score=None) -> Tensor",
     # post-normed stream, query/key norms with rotated values, decayed linear attention, experts with weights on their outputs
     "attn_prep_store": "(Tensor x, int q_off, int k_off, int v_off, Tensor positions, Tensor? q_w, Tensor? k_w, str norm_mode, float eps, "
                        "Tensor? freq, int rot_dims, bool interleaved, Tensor? vfreq, Tensor? slots, Tensor(a!)? k_cache, Tensor(b!)? v_cache, "
@@ -102,6 +103,17 @@ _DEFS = {
     "moe_glu": "(Tensor gu, float limit, float alpha, float shift=1.0) -> Tensor",
     "moe_gather_rows": "(Tensor ys, Tensor dst, Tensor? wts=None) -> Tensor",
     "skinny_proj": "(Tensor x, Tensor w, str in_act) -> Tensor",
+    # several residual streams, the real-gated recurrence, a latent with a rotated key part, the softmax router with groups
+    "hyper_mix": "(Tensor(a!) x, Tensor? y, Tensor? scale, Tensor? mix, Tensor? w_out, Tensor? w_in, Tensor? w_norm, float eps, ScalarType out_dtype) "
+                 "-> Tensor",
+    "hyper_start": "(Tensor x, int n_streams, Tensor? w_in, Tensor? w_norm, float eps, ScalarType out_dtype) -> (Tensor, Tensor)",
+    "short_conv": "(Tensor x, Tensor w, Tensor(a!)? state, Tensor pos0, Tensor state_slot, Tensor? qo_indptr, Tensor? tok_seq, Tensor? bias, "
+                  "str act) -> Tensor",
+    "rglru_scan": "(Tensor y, Tensor u, Tensor gates, Tensor gate_bias, Tensor rate, Tensor(a!) state, Tensor pos0, Tensor state_slot, "
+                  "Tensor? qo_indptr, Tensor? tok_seq) -> Tensor",
+    "latent_rope_prep": "(Tensor x, int q_off, int kv_off, int g_off, Tensor positions, Tensor? freq, float mag, Tensor w_kv, float eps, "
+                        "Tensor slots, Tensor(a!) cache, int heads, int dim, int rot) -> (Tensor, Tensor)",
+    "moe_route_softmax": "(Tensor logits, int top, int n_groups, int keep_groups, float norm_eps) -> (Tensor, Tensor)",
 }
 for _name, _sig in _DEFS.items():
     _LIB.define(_name + _sig)
@@ -296,9 +308,10 @@ def _rope_vnorm_store(qkv, positions, freq, mag, rot_dims, eps, slots, k_cache, 
 
 
 def _softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, pos0, state_slot, qo_indptr, tok_seq, scale, cap, heads, kv_heads, dim, vdim,
-                  window=0, r1=None, r2=None, v_turn=None, v_interleaved=False, gate=None):
+                  window=0, r1=None, r2=None, v_turn=None, v_interleaved=False, gate=None, sink_score=None):
     return ops.softcap_attn(q, k_cache, v_cache, kv_indices, kv_start, kv_len, _layout(q.shape[0], pos0, state_slot, qo_indptr, tok_seq), scale, cap,
-                            heads, kv_heads, dim, vdim, window=window, r1=r1, r2=r2, v_turn=v_turn, v_interleaved=v_interleaved, gate=gate)
+                            heads, kv_heads, dim, vdim, window=window, r1=r1, r2=r2, v_turn=v_turn, v_interleaved=v_interleaved, gate=gate,
+                            sink_score=sink_score)
 
 
 def _attn_prep_store(x, q_off, k_off, v_off, positions, q_w, k_w, norm_mode, eps, freq, rot_dims, interleaved, vfreq, slots, k_cache, v_cache,
@@ -349,6 +362,30 @@ def _moe_gather_rows(ys, dst, wts=None):
 
 def _skinny_proj(x, w, in_act):
     return ops.skinny_proj(x, w, in_act)
+
+
+def _hyper_mix(x, y, scale, mix, w_out, w_in, w_norm, eps, out_dtype):
+    return ops.hyper_mix(x, y, scale, mix, w_out, w_in, w_norm, eps, out_dtype=out_dtype)[1]
+
+
+def _hyper_start(x, n_streams, w_in, w_norm, eps, out_dtype):
+    return ops.hyper_mix(x, w_in=w_in, w_norm=w_norm, eps=eps, n_streams=n_streams, out_dtype=out_dtype)
+
+
+def _short_conv(x, w, state, pos0, state_slot, qo_indptr, tok_seq, bias, act):
+    return ops.short_conv(x, w, state, _layout(x.shape[0], pos0, state_slot, qo_indptr, tok_seq), bias=bias, act=act)
+
+
+def _rglru_scan(y, u, gates, gate_bias, rate, state, pos0, state_slot, qo_indptr, tok_seq):
+    return ops.rglru_scan(y, u, gates, gate_bias, rate, state, _layout(u.shape[0], pos0, state_slot, qo_indptr, tok_seq))
+
+
+def _latent_rope_prep(x, q_off, kv_off, g_off, positions, freq, mag, w_kv, eps, slots, cache, heads, dim, rot):
+    return ops.latent_rope_prep(x, (q_off, kv_off, g_off), positions, freq, mag, w_kv, eps, slots, cache, heads, dim, rot)
+
+
+def _moe_route_softmax(logits, top, n_groups, keep_groups, norm_eps):
+    return ops.moe_route_softmax(logits, top, n_groups, keep_groups, norm_eps)
 
 
 for _name in _DEFS:

@@ -115,7 +115,9 @@ def test_every_kernel_entry_point_has_a_custom_op():
              "nvx_rope_vnorm_store": "rope_vnorm_store", "nvx_softcap_attn": "softcap_attn", "nvx_moe_route": "moe_route",
              "nvx_moe_expert_rows": "moe_expert_rows", "nvx_moe_scatter_rows": "moe_scatter_rows", "nvx_moe_order": "moe_order", "nvx_moe_glu": "moe_glu",
              "nvx_moe_gather_rows": "moe_gather_rows", "nvx_skinny_proj": "skinny_proj", "nvx_attn_prep_store": "attn_prep_store",
-             "nvx_decay_scan": "decay_scan", "nvx_postnorm_residual": "postnorm_residual", "nvx_embed_scale": "embed_scale", "nvx_tanh_cap": "tanh_cap"}
+             "nvx_decay_scan": "decay_scan", "nvx_postnorm_residual": "postnorm_residual", "nvx_embed_scale": "embed_scale", "nvx_tanh_cap": "tanh_cap",
+             "nvx_hyper_mix": "hyper_mix", "nvx_short_conv": "short_conv", "nvx_rglru_scan": "rglru_scan", "nvx_latent_rope_prep": "latent_rope_prep",
+             "nvx_moe_route_softmax": "moe_route_softmax"}
     helpers = {"nvx_abi_version", "nvx_last_error", "nvx_linear_decode_splits", "nvx_decode_plan_ws_ints", "nvx_decode_partial_ws_floats",
                "nvx_prefill_plan_ws_ints", "nvx_sample_ws_bytes", "nvx_paged_decode_noalloc_max_batch",
                "nvx_lmhead_max_rows", "nvx_lmhead_rows_per_pass", "nvx_lmhead_packed_elems", "nvx_lmhead_ws_bytes",
