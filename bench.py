@@ -805,9 +805,177 @@ def _gibavik_kernel_table(z, t_pre, n_dec, ctx, phases=("prefill", "decode")):
     return rows
 
 
+def _ladusun_config(z):
+    """Layers attention, rglru, latent_attention in turn, the second attention layer reading the first one's keys and values; heads of
+    128 with 8 key/value heads and 64 rotated dimensions; a latent of at most 448 with a rotated key part of 64 (cache rows of 320 or
+    512); recurrences as wide as the model in blocks of 128 channels behind four taps; four streams; the first feed-forward dense
+    (two matrices, so 3/2 of the gated model's size), the others eight experts of ff / 2 in four groups, two a token."""
+    w = z["width"]
+    bands = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}
+    ramp = {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}
+    dense = {"kind": "dense", "ff": z["ff"] * 3 // 2}
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 2, "limit": 7.0}, "router": {"experts": 8, "top": 2, "groups": {"count": 4, "keep": 2}}}
+    att = {"type": "attention", "mixer": {"heads": z["heads"], "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5, "softcap": 30.0,
+                                          "rot": {"dims": 64, "base": 5e5, "scaling": bands}}}
+    lat = {"type": "latent_attention", "mixer": {"heads": z["heads"], "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": min(z["kv_rank"], 448),
+                                                 "scale": 192 ** -0.5, "rot": {"dims": 64, "base": 1e4, "scaling": ramp}}}
+    rec = {"type": "rglru", "mixer": {"width": w, "blocks": w // 128, "conv": 4}}
+    layers = []
+    for i in range(z["layers"]):
+        layer = json.loads(json.dumps((att, rec, lat)[i % 3]))
+        layer["mlp"] = dense if i == 0 else moe
+        if i == 3:
+            layer["mixer"]["kv_from"] = 0
+        layers.append(layer)
+    return {"architecture": "Ladusun", "vocab": z["vocab"], "width": w, "norm": {"eps": 1e-5}, "embedding": {"scale": 8.0}, "streams": 4,
+            "layers": layers}
+
+
+def _ladusun_kernel_table(z, t_pre, n_dec, ctx, phases=("prefill", "decode")):
+    """Each kernel of Ladusun beside the like kernel of Gibavik, Kabidra, Meronex or Qwen3 at the same shape: time, and the fraction of
+    its roofline (HBM bytes it must move at 8 TB/s; attention in prefill: its multiply-adds at the dense bf16 MFMA peak)."""
+    from nano_vllm_x_amd import ops
+    from nano_vllm_x_amd.layers.latent_attention import RotaryLatentAttention
+    from nano_vllm_x_amd.layers.rotary_embedding import rotary_frequencies
+    dev, bf = torch.device("cuda"), torch.bfloat16
+    w, ff, h, streams = z["width"], z["ff"] // 2, z["heads"], 4
+    rank = min(z["kv_rank"], 448)
+    row = RotaryLatentAttention.padded_row(rank + 64)
+    rows = []
+
+    def layout(n_seq, q_len, pos0):
+        p = torch.full((n_seq,), pos0, dtype=torch.int64, device=dev)
+        sl = torch.arange(n_seq, dtype=torch.int32, device=dev)
+        if q_len == 1:
+            return ops.StepLayout(n_seq, n_seq, p, sl)
+        qo = torch.arange(0, n_seq + 1, dtype=torch.int32, device=dev) * q_len
+        return ops.StepLayout(n_seq * q_len, n_seq, p, sl, qo, torch.arange(n_seq, dtype=torch.int32, device=dev).repeat_interleave(q_len))
+
+    def add(name, phase, us, bytes_=None, flops=None, like=None):
+        if bytes_:
+            frac, bound = bytes_ / (us * 1e-6) / (HBM_PEAK_GBS * 1e9), "HBM"
+        else:
+            frac, bound = flops / (us * 1e-6) / (MFMA_BF16_PEAK_TFLOPS * 1e12), "MFMA"
+        rows.append({"kernel": name, "phase": phase, "us": round(us, 1), "of_roofline": round(frac, 3), "bound": bound, "like": like})
+
+    for phase, (n_seq, q_len, pos0) in (("prefill", (max(t_pre // 1024, 1), 1024, 0)), ("decode", (n_dec, 1, ctx))):
+        if phase not in phases:
+            continue
+        t = n_seq * q_len
+        dec = phase == "decode"
+        lay = layout(n_seq, q_len, pos0)
+        reps = 20 if dec else 3
+        y, x1 = torch.randn(t, w, device=dev).to(bf), torch.randn(t, w, device=dev)
+        xs = torch.randn(t, streams, w, device=dev)
+        wv, one = torch.ones(w, device=dev), torch.ones(1, device=dev)
+        a_s, mix = torch.full((streams,), 0.5, device=dev), torch.eye(streams, device=dev)
+        # sublayer boundary over four streams: reads the result (2 B) and the streams (4 x 4 B), writes the streams (4 x 4 B) and the
+        # rows the next sublayer reads (2 B); the one-stream kernels read and write 4 B of stream
+        add("hyper_mix (4 streams)", phase, _time_us(lambda: ops.hyper_mix(xs, y, scale=wv, mix=mix, w_out=a_s, w_in=a_s, w_norm=wv, eps=1e-5)),
+            bytes_=t * w * (4 + 8 * streams), like="postnorm_residual / rmsnorm+residual")
+        add("gibavik postnorm_residual (1 stream)", phase, _time_us(lambda: ops.postnorm_residual(x1, y=y, w_post=one, eps=1e-5)), bytes_=t * w * 12)
+        xb = x1.to(bf)
+        add("qwen3 rmsnorm+residual (1 stream, 16-bit)", phase, _time_us(lambda: ops.rmsnorm(y, wv.to(bf), 1e-5, xb)), bytes_=t * w * 8)
+        # dense feed-forward activation, and the experts'
+        up = torch.randn(t, 3 * ff, device=dev).to(bf)
+        add("relu2", phase, _time_us(lambda: ops.relu2(up)), bytes_=t * 3 * ff * 4, like="silu_mul")
+        gu = torch.randn(t, 2 * ff, device=dev).to(bf)
+        add("moe_glu (limit, 1.702, u + 1)", phase, _time_us(lambda: ops.moe_glu(gu, 7.0, 1.702, 1.0)), bytes_=t * ff * 6, like="silu_mul")
+        add("qwen3 silu_mul", phase, _time_us(lambda: ops.silu_mul(gu)), bytes_=t * ff * 6)
+        # router: eight experts in four groups, two a token
+        z8 = torch.randn(t, 8, device=dev)
+        add("moe_route_softmax (groups)", phase, _time_us(lambda: ops.moe_route_softmax(z8, 2, 4, 2, 1e-20)), bytes_=t * (8 * 4 + 2 * 8), like="moe_route")
+        add("meronex moe_route", phase, _time_us(lambda: ops.moe_route(z8, 2)), bytes_=t * (8 * 4 + 2 * 8))
+        # recurrence: convolution of four taps with a bias, then the gated scan (reads y, u, two gates: 2 B each; writes 2 B)
+        yx = torch.randn(t, 2 * w, device=dev).to(bf)
+        taps, cb = torch.randn(4, w, device=dev), torch.randn(w, device=dev)
+        cst = torch.zeros(n_seq + 1, 3, w, device=dev)
+        add("short_conv (bias)", phase, _time_us(lambda: ops.short_conv(yx[:, w:], taps, cst, lay, bias=cb)), bytes_=t * w * 4 + n_seq * 3 * w * 8,
+            like="canon_conv / short_conv_silu")
+        add("meronex short_conv_silu", phase, _time_us(lambda: ops.short_conv_silu(yx[:, w:], taps, cst, lay)), bytes_=t * w * 4 + n_seq * 3 * w * 8)
+        u = torch.randn(t, w, device=dev).to(bf)
+        gates = torch.randn(w // 128, t, 256, device=dev).to(bf)
+        gb, rate = torch.zeros(2, w, device=dev), torch.full((w,), 0.05, device=dev)
+        st = torch.zeros(n_seq + 1, w, device=dev)
+        add("rglru_scan", phase, _time_us(lambda: ops.rglru_scan(yx[:, :w], u, gates, gb, rate, st, lay), reps), bytes_=t * w * 10 + n_seq * w * 8,
+            like="mingru_scan")
+        zxg = torch.randn(t, 3 * w, device=dev).to(bf)
+        add("kabidra mingru_scan", phase, _time_us(lambda: ops.mingru_scan(zxg, st, lay), reps), bytes_=t * w * 8 + n_seq * w * 8)
+        # attention: 8 key/value heads of 128, beside paged attention over the same tokens
+        kv_len = pos0 + q_len
+        n_rows = n_seq * kv_len
+        kc, vc = torch.randn(n_rows, 8 * 128, device=dev).to(bf), torch.randn(n_rows, 8 * 128, device=dev).to(bf)
+        idx = torch.arange(n_rows, dtype=torch.int32, device=dev)
+        kv_start = torch.arange(n_seq, dtype=torch.int64, device=dev) * kv_len
+        kvl = torch.full((n_seq,), kv_len, dtype=torch.int32, device=dev)
+        qkv = torch.randn(t, (h + 16) * 128 + h, device=dev).to(bf)          # q | k | v | one gate per head
+        pos = (torch.arange(t, device=dev) % q_len + pos0).to(torch.int64)
+        slots = (torch.arange(t, device=dev) // q_len * kv_len + pos).to(torch.int64)
+        fr = rotary_frequencies(64, 5e5, {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192})[0].to(dev)
+        prep_bytes = t * (h + 16) * 128 * 2 * 2
+        add("attn_prep_store (rotation in neighbouring pairs, no norms)", phase,
+            _time_us(lambda: ops.attn_prep_store(qkv, (0, h * 128, (h + 8) * 128), pos, None, None, "none", 1e-5, fr, 64, True, None, slots, kc, vc, h, 8, 128, 128)),
+            bytes_=prep_bytes, like="attn_prep_store (head norms)")
+        qn = torch.ones(128, device=dev)
+        add("gibavik attn_prep_store (head norms, rotation)", phase,
+            _time_us(lambda: ops.attn_prep_store(qkv, (0, h * 128, (h + 8) * 128), pos, qn, qn, "head", 1e-5, fr, 64, False, None, slots, kc, vc, h, 8, 128, 128)),
+            bytes_=prep_bytes)
+        q128 = torch.randn(t, h * 128, device=dev).to(bf)
+        g_h = qkv[:, (h + 16) * 128:]
+        us_sink = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 30.0, h, 8, 128, 128, gate=g_h, sink_score=0.0), reps)
+        us_plain = _time_us(lambda: ops.softcap_attn(q128, kc, vc, idx, kv_start, kvl, lay, 0.09, 30.0, h, 8, 128, 128), reps)
+        kc4, vc4 = kc.view(n_rows, 8, 128), vc.view(n_rows, 8, 128)
+        # latent attention over rows of [latent | rotated key part]
+        lfr, mag = rotary_frequencies(64, 1e4, {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0})
+        lfr = lfr.to(dev)
+        xl = torch.randn(t, h * 192 + rank + 64 + h, device=dev).to(bf)
+        pool = torch.randn(n_rows, row, device=dev).to(bf)
+        add("latent_rope_prep", phase,
+            _time_us(lambda: ops.latent_rope_prep(xl, (0, h * 192, h * 192 + rank + 64), pos, lfr, mag, wv[:rank].contiguous(), 1e-5, slots, pool, h, 128, 64)),
+            bytes_=t * (h * 192 * 2 + rank + 64 + row) * 2, like="attn_prep_store")
+        qf = torch.randn(h, t, row, device=dev).to(bf)
+        gl = torch.rand(t, h, device=dev)
+        us_lat = _time_us(lambda: ops.latent_attn(qf, pool, idx, kv_start, kvl, lay, 0.07, gate=gl), reps)
+        r2 = 256 if row <= 320 else 512
+        pool2, qf2 = torch.randn(n_rows, r2, device=dev).to(bf), torch.randn(h, t, r2, device=dev).to(bf)
+        us_lat2 = _time_us(lambda: ops.latent_attn(qf2, pool2, idx, kv_start, kvl, lay, 0.07), reps)
+        if not dec:
+            pairs = n_seq * q_len * (q_len + 1) // 2
+            add("softcap_attn (silent term, one gate per head)", phase, us_sink, flops=4.0 * h * 128 * pairs, like="paged_prefill")
+            add("meronex softcap_attn (capped scores only)", phase, us_plain, flops=4.0 * h * 128 * pairs)
+            add(f"latent_attn (rows of {row}, gates)", phase, us_lat, flops=4.0 * h * row * pairs, like="paged_prefill")
+            add(f"kabidra latent_attn (rows of {r2})", phase, us_lat2, flops=4.0 * h * r2 * pairs)
+            plan = ops.prefill_plan_ws(n_seq, dev)
+            kv_indptr = torch.arange(0, n_seq + 1, dtype=torch.int32, device=dev) * kv_len
+            ops.prefill_plan(lay.qo_indptr, plan)
+            us = _time_us(lambda: ops.paged_prefill(q128, kc4, vc4, lay.qo_indptr, kv_indptr, idx, plan, h, 8, 0.1), reps=5)
+            add("qwen3 paged_prefill", phase, us, flops=4.0 * h * 128 * pairs)
+        else:
+            io = 2 * t * h * 128 * 2
+            add("softcap_attn (silent term, one gate per head)", phase, us_sink, bytes_=n_rows * 8 * 128 * 2 * 2 + io, like="paged_decode")
+            add("meronex softcap_attn (capped scores only)", phase, us_plain, bytes_=n_rows * 8 * 128 * 2 * 2 + io)
+            add(f"latent_attn (rows of {row}, gates)", phase, us_lat, bytes_=n_rows * row * 2 + 2 * t * h * row * 2, like="paged_decode")
+            add(f"kabidra latent_attn (rows of {r2})", phase, us_lat2, bytes_=n_rows * r2 * 2 + 2 * t * h * r2 * 2)
+            ws = ops.DecodeWorkspace(n_seq, h, 8, dev)
+            ops.decode_plan(kvl, kv_start, ws)
+            us = _time_us(lambda: ops.paged_decode(q128, kc4, vc4, idx, n_seq, ws, 0.1))
+            add("qwen3 paged_decode", phase, us, bytes_=n_rows * 8 * 128 * 2 * 2 + io)
+            # experts: eight of ff / 2, two a token, the weights on the outputs
+            hm = torch.randn(t, w, device=dev).to(bf)
+            w_gu, w_d = torch.randn(8, 2 * ff, w, device=dev).to(bf) * 0.02, torch.randn(8, w, ff, device=dev).to(bf) * 0.02
+            eidx = torch.stack([torch.randperm(8, device=dev)[:2] for _ in range(t)]).to(torch.int32)
+            wts = torch.full((t, 2), 0.5, device=dev)
+            us = _time_us(lambda: ops.moe_expert_rows(hm, eidx, wts, w_gu, w_d, 7.0, 1.702, 1.0, True))
+            add("moe_expert_rows (limit, weights on outputs)", phase, us, bytes_=min(t * 2, 8) * 3 * ff * w * 2, like="gibavik moe_expert_rows")
+            us = _time_us(lambda: ops.moe_expert_rows(hm, eidx, wts, w_gu, w_d, float("inf"), 1.0, 0.0, True))
+            add("gibavik moe_expert_rows", phase, us, bytes_=min(t * 2, 8) * 3 * ff * w * 2)
+    return rows
+
+
 ARCHS = {"kabidra": (lambda z: _kabidra_config(z), lambda *a, **k: _kernel_table(*a), "Kabidra"),
          "meronex": (lambda z: _meronex_config(z), lambda *a, **k: _meronex_kernel_table(*a, **k), "Meronex"),
-         "gibavik": (lambda z: _gibavik_config(z), lambda *a, **k: _gibavik_kernel_table(*a, **k), "Gibavik")}
+         "gibavik": (lambda z: _gibavik_config(z), lambda *a, **k: _gibavik_kernel_table(*a, **k), "Gibavik"),
+         "ladusun": (lambda z: _ladusun_config(z), lambda *a, **k: _ladusun_kernel_table(*a, **k), "Ladusun")}
 
 
 def arch_compare(args):
@@ -829,7 +997,10 @@ def arch_compare(args):
         z = ARCH_SIZES[name]
         entry = {"geometry": z}
         with tempfile.TemporaryDirectory() as tmp:
-            for model, cfg in ((args.arch, make_config(z)), ("qwen3", _qwen3_config(z))) if args.arch_serve else ():
+            engines = [(args.arch, make_config(z)), ("qwen3", _qwen3_config(z))]
+            if args.arch == "ladusun":          # its closest relative in this package (attention with borrowed keys beside a recurrence, experts)
+                engines.insert(1, ("gibavik", _gibavik_config(z)))
+            for model, cfg in engines if args.arch_serve else ():
                 d = os.path.join(tmp, model)
                 os.makedirs(d)
                 with open(os.path.join(d, "config.json"), "w") as f:
@@ -843,7 +1014,7 @@ def arch_compare(args):
         print(f"[arch-compare] {name}: kernels one by one", file=sys.stderr, flush=True)
         with torch.inference_mode():
             t_pre = args.arch_seqs * args.arch_prompt
-            if args.arch == "gibavik" and args.arch_portion:      # the kernels one by one at the size of the steps the engines ran
+            if args.arch in ("gibavik", "ladusun") and args.arch_portion:      # the kernels one by one at the size of the steps the engines ran
                 t_pre = min(t_pre, max(args.arch_portion, args.arch_prompt))
             entry["kernels"] = kernel_table(z, t_pre, args.arch_seqs, args.arch_prompt,
                                             phases=tuple(args.arch_phases.split(",")))

@@ -84,6 +84,19 @@ def attention_frequencies(m):
     return plain_frequencies(rot["dims"], rot["base"]), 1.0
 
 
+def sink_softmax_readout(q, k, v, pos_q, pos_k, scale, cap=None, sink=0.0):
+    """One head: q (T, dim) at positions pos_q over keys k (S, dim), values v (S, vdim) at positions pos_k.  Scores scale * q . k
+    pass cap * tanh(. / cap); key j counts for query i when pos_k[j] <= pos_q[i]; the weights are exp(score) over
+    exp(sink) + the sum of the visible ones (sink None: over the sum alone), so they add up to less than one."""
+    s = (q @ k.T) * scale
+    if cap:
+        s = cap * torch.tanh(s / cap)
+    seen = pos_q[:, None] >= pos_k[None, :]
+    e = torch.where(seen, torch.exp(s), torch.zeros_like(s))
+    extra = 0.0 if sink is None else math.exp(sink)
+    return (e / (extra + e.sum(-1, keepdim=True))) @ v
+
+
 def sink_attention(h, w, p, m, pos, kv):
     """Grouped-head attention with capped scores, a silent extra term of score 0 in the softmax's denominator, and one sigmoid
     gate per head.  `kv` = (keys, values) as attention_keys_values makes them (this layer's, or a lender's)."""
@@ -93,15 +106,8 @@ def sink_attention(h, w, p, m, pos, kv):
     q = turn_pairs(q, pos, *attention_frequencies(m))
     keys, values = kv
     gate = torch.sigmoid(h @ w[p + "g"].T)                                   # (T, heads)
-    causal = pos[:, None] >= pos[None, :]
-    heads = []
-    for j in range(hq):
-        k, v = keys[:, j // (hq // g)], values[:, j // (hq // g)]
-        s = (q[j] @ k.T) * m["scale"]
-        if m.get("softcap"):
-            s = m["softcap"] * torch.tanh(s / m["softcap"])
-        e = torch.where(causal, torch.exp(s), torch.zeros_like(s))
-        heads.append((e / (1.0 + e.sum(-1, keepdim=True))) @ v * gate[:, j:j + 1])
+    heads = [sink_softmax_readout(q[j], keys[:, j // (hq // g)], values[:, j // (hq // g)], pos, pos, m["scale"], m.get("softcap")) * gate[:, j:j + 1]
+             for j in range(hq)]
     return torch.cat(heads, -1) @ w[p + "o"].T + w[p + "o.b"]
 
 
@@ -128,6 +134,26 @@ def latent_attention(h, w, p, m, pos, eps):
     return torch.cat(heads, -1) @ w[p + "o"].T
 
 
+def causal_conv(x, taps, bias):
+    """x (T, channels); taps (channels, n) whose last column multiplies the current token; zeros stand before the first token."""
+    t, n = x.shape[0], taps.shape[1]
+    padded = torch.cat([torch.zeros(n - 1, x.shape[1], dtype=x.dtype), x])
+    return bias + sum(padded[j:j + t] * taps[:, j] for j in range(n))
+
+
+def gated_recurrence(u, r_pre, i_pre, lam, start=None):
+    """S_t = a_t S_(t-1) + sqrt(1 - a_t^2) sigmoid(i_pre_t) u_t with a_t = exp(-8 sigmoid(r_pre_t) softplus(lam)), every channel on
+    its own, from `start` (zeros if None).  Returns all S_t (T, channels)."""
+    a = torch.exp(-8.0 * torch.sigmoid(r_pre) * torch.nn.functional.softplus(lam))
+    b = torch.sqrt(1.0 - a * a) * torch.sigmoid(i_pre) * u
+    state = torch.zeros_like(u[0]) if start is None else start
+    out = []
+    for n in range(u.shape[0]):
+        state = a[n] * state + b[n]
+        out.append(state)
+    return torch.stack(out)
+
+
 def rglru(h, w, p, m):
     """Two branches: a gelu gate, and a per-channel causal convolution followed by a diagonal recurrence whose decay and input gate
     are sigmoids of block-diagonal maps of the convolved branch."""
@@ -135,20 +161,12 @@ def rglru(h, w, p, m):
     width, blocks, taps = m["width"], m["blocks"], m["conv"]
     y = gelu_tanh(h @ w[p + "y"].T + w[p + "y.b"])
     x = h @ w[p + "x"].T + w[p + "x.b"]
-    padded = torch.cat([torch.zeros(taps - 1, width, dtype=F64), x])
-    u = w[p + "conv.b"] + sum(padded[j:j + t] * w[p + "conv"][:, j] for j in range(taps))
+    u = causal_conv(x, w[p + "conv"], w[p + "conv.b"])
     bw = width // blocks
     ub = u.view(t, blocks, bw)
-    r = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, w[p + "ra"]) + w[p + "ra.b"]).reshape(t, width)
-    i = torch.sigmoid(torch.einsum("tbi,boi->tbo", ub, w[p + "ri"]) + w[p + "ri.b"]).reshape(t, width)
-    a = torch.exp(-8.0 * r * torch.nn.functional.softplus(w[p + "lam"]))
-    b = torch.sqrt(1.0 - a * a) * i * u
-    state = torch.zeros(width, dtype=F64)
-    out = []
-    for n in range(t):
-        state = a[n] * state + b[n]
-        out.append(state)
-    return (torch.stack(out) * y) @ w[p + "o"].T
+    r = (torch.einsum("tbi,boi->tbo", ub, w[p + "ra"]) + w[p + "ra.b"]).reshape(t, width)
+    i = (torch.einsum("tbi,boi->tbo", ub, w[p + "ri"]) + w[p + "ri.b"]).reshape(t, width)
+    return (gated_recurrence(u, r, i, w[p + "lam"]) * y) @ w[p + "o"].T
 
 
 def dense_ff(h, w, p):
@@ -158,8 +176,12 @@ def dense_ff(h, w, p):
 def route(h, w, p, router):
     """(ids, weights) per token: softmax over all experts, experts outside the best groups struck out, the `top` largest kept and
     their scores divided by their sum."""
+    return route_logits(h @ w[p + "router"].T, router)
+
+
+def route_logits(z, router):
     n, top = router["experts"], router["top"]
-    s = torch.softmax(h @ w[p + "router"].T, -1)
+    s = torch.softmax(z, -1)
     groups = router.get("groups")
     allowed = torch.ones_like(s, dtype=torch.bool)
     if groups:
@@ -188,6 +210,17 @@ def moe_ff(h, w, p, mlp):
     return out
 
 
+def read_streams(xs, a_in):
+    """What a sublayer reads of the streams xs (a list of (T, width)): sum_s a_in[s] xs[s]."""
+    return sum(a_in[s] * xs[s] for s in range(len(xs)))
+
+
+def move_streams(xs, y, mix, a_out):
+    """All streams at once from the old ones: stream t becomes sum_s mix[s, t] xs[s] + a_out[t] y."""
+    n = len(xs)
+    return [sum(mix[s, t] * xs[s] for s in range(n)) + a_out[t] * y for t in range(n)]
+
+
 def forward(cfg: dict, weights: dict, tokens, layer_sums: list | None = None):
     """Logits (T, vocab) of one sequence computed whole.  `layer_sums`, a list, receives the sum of the streams after every layer."""
     w = {k: (v.to(F64) if v.is_floating_point() else v) for k, v in weights.items()}
@@ -201,14 +234,12 @@ def forward(cfg: dict, weights: dict, tokens, layer_sums: list | None = None):
     def sublayer(q, p, fn):
         nonlocal xs
         hyper = (p + f"hc{q}.in") in w
-        a_in = w[p + f"hc{q}.in"] if hyper else torch.ones(1, dtype=F64)
-        u = sum(a_in[s] * xs[s] for s in range(n_streams))
+        u = read_streams(xs, w[p + f"hc{q}.in"]) if hyper else xs[0]
         y = fn(rms(u, eps) * w[p + f"norm{q}"])
         if (p + f"ls{q}") in w:
             y = y * w[p + f"ls{q}"]
         if hyper:
-            mix, a_out = w[p + f"hc{q}.mix"], w[p + f"hc{q}.out"]
-            xs = [sum(mix[s, t] * xs[s] for s in range(n_streams)) + a_out[t] * y for t in range(n_streams)]
+            xs = move_streams(xs, y, w[p + f"hc{q}.mix"], w[p + f"hc{q}.out"])
         else:
             xs = [xs[0] + y]
 

@@ -1,0 +1,672 @@
+"""Ladusun through the engine, and its kernels alone, against the plain restatement in oracle/ladusun_oracle.py.
+
+Every test makes its own small configuration and weights.  The engine is built on a directory that holds config.json (and,
+where the weights are made by the test, model.safetensors), as a user's would be; steps are given with Engine.run_given (the
+replay entry point) or chosen by the scheduler (Engine.step / LLM.generate).  Comparisons are in float32 unless a test says
+otherwise: there a structural fault (a key too many, a lost state, a silent softmax term left out) stands far above rounding.
+"""
+import asyncio
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import ladusun_oracle as lo
+from seq_drivers import F32_TOL, close, cuts_of, greedy, make_engine, model_dir, replay, step_layout, tokens
+
+pytestmark = pytest.mark.gpu
+
+BANDS = {"factor": 3.0, "low": 0.5, "high": 4.0, "original": 64}           # with base 300 over 8 dimensions: one pair kept, two blended, one stretched
+RAMP = {"factor": 2.5, "original": 48, "fast": 4.0, "slow": 0.5}           # with base 200 over 6 dimensions: ramp 0, 1/2, 1
+DENSE = {"kind": "dense", "ff": 50}
+MOE = {"kind": "moe", "expert": {"ff": 16, "limit": 1.5}, "router": {"experts": 6, "top": 3, "groups": {"count": 3, "keep": 2}}}
+MOE1 = {"kind": "moe", "expert": {"ff": 10, "limit": 0.8}, "router": {"experts": 4, "top": 1}}
+ATT = {"type": "attention", "mixer": {"heads": 6, "kv_heads": 2, "dim": 12, "vdim": 20, "scale": 0.3, "softcap": 5.0,
+                                      "rot": {"dims": 8, "base": 300.0, "scaling": BANDS}}, "mlp": DENSE}
+LAT = {"type": "latent_attention", "mixer": {"heads": 3, "dim": 10, "rot_dim": 6, "vdim": 14, "kv_rank": 9, "scale": 0.25,
+                                             "rot": {"dims": 6, "base": 200.0, "scaling": RAMP}}, "mlp": MOE}
+REC = {"type": "rglru", "mixer": {"width": 24, "blocks": 3, "conv": 4}, "mlp": MOE1}
+
+
+def borrowing(layer, src, mlp=MOE1, **changes):
+    return {"type": "attention", "mixer": dict(layer["mixer"], kv_from=src, **changes), "mlp": mlp}
+
+
+def make_cfg(layers, width=40, vocab=61, eps=1e-5, emb=3.0, streams=3):
+    cfg = {"architecture": "Ladusun", "vocab": vocab, "width": width, "norm": {"eps": eps}, "embedding": {"scale": emb},
+           "layers": json.loads(json.dumps(layers))}
+    if streams is not None:
+        cfg["streams"] = streams
+    return cfg
+
+
+def weights_of(cfg, seed=0):
+    """The weights an engine built on a directory without a checkpoint draws for `seed`."""
+    from nano_vllm_x_amd.ladusun import LadusunConfig, random_checkpoint
+    return dict(random_checkpoint(LadusunConfig.from_dict(cfg), seed))
+
+
+def sharpen(w, by=3.0, names=("mix.q", "mix.k", "mix.dkv")):
+    """Peaked attention scores: one key too many or too few then moves the result far."""
+    for name in w:
+        if name.endswith(names):
+            w[name] = (w[name] * by).to(torch.bfloat16).float()
+    return w
+
+
+def forward(cfg, w, toks):
+    return lo.forward(cfg, w, toks)
+
+
+# ---- kernels alone -------------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("fmt", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("streams,width", [(1, 70), (3, 1), (5, 300), (2, 64), (9, 33)])
+def test_streams_move_together_at_a_sublayer_boundary(fmt, streams, width):
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(streams * 1000 + width)
+    t, eps = 5, 1e-3 if width > 1 else 1.0          # a row of one number is its own sign once it is normed, unless eps counts
+    rnd = lambda *s: torch.randn(*s, generator=g)
+    tol = 1e-5 if fmt == torch.float32 else 4e-2
+    # the start: every stream is the one row of its token; what the first sublayer reads
+    x0, a_in, wn = rnd(t, width), rnd(streams), rnd(width)
+    x, h = ops.hyper_mix(x0.cuda(), w_in=a_in.cuda(), w_norm=wn.cuda(), eps=eps, n_streams=streams, out_dtype=fmt)
+    assert x.shape == (t, streams, width) and x.dtype == torch.float32 and h.dtype == fmt
+    assert torch.equal(x.cpu(), x0[:, None, :].expand(t, streams, width))
+    close(h.float().cpu(), lo.rms(lo.read_streams([x0.double()] * streams, a_in.double()), eps) * wn.double(), tol, "first read")
+    # a boundary between two sublayers, on streams that differ: layer scale, all streams from the old ones, the next read
+    xs = [rnd(t, width) for _ in range(streams)]
+    y, ls, mix, a_out, a_in2, wn2 = rnd(t, width).to(fmt), rnd(width), rnd(streams, streams), rnd(streams), rnd(streams), rnd(width)
+    xd = torch.stack(xs, 1).cuda()
+    x2, h2 = ops.hyper_mix(xd, y.cuda(), scale=ls.cuda(), mix=mix.cuda(), w_out=a_out.cuda(), w_in=a_in2.cuda(), w_norm=wn2.cuda(), eps=eps)
+    want = lo.move_streams([a.double() for a in xs], y.double() * ls.double(), mix.double(), a_out.double())
+    assert x2.data_ptr() == xd.data_ptr()
+    close(x2.cpu(), torch.stack(want, 1), 1e-5, "streams")
+    close(h2.float().cpu(), lo.rms(lo.read_streams(want, a_in2.double()), eps) * wn2.double(), tol, "next read")
+    # a transposed mixing matrix is another function (the matrix is [from, to])
+    if streams > 1:
+        other = lo.move_streams([a.double() for a in xs], y.double() * ls.double(), mix.double().T, a_out.double())
+        assert (torch.stack(other, 1) - torch.stack(want, 1)).abs().max() > 0.1
+    # the end: the streams stay, their plain sum is normed
+    before = x2.clone()
+    x3, h3 = ops.hyper_mix(x2, w_norm=wn.cuda(), eps=eps, out_dtype=fmt)
+    assert torch.equal(x3, before)
+    close(h3.float().cpu(), lo.rms(sum(want), eps) * wn.double(), tol, "closing norm of the sum")
+
+
+def test_latent_rows_are_normed_rotated_and_stored():
+    """Positions up to several thousand; the parts are slices of a wider projection; a negative slot stores nothing; the cache row is
+    longer than the latent and the key part, and its tail is cleared."""
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(5)
+    t, heads, dim, rot, rank, row, eps = 6, 3, 10, 6, 9, 32, 1e-4
+    hq = heads * (dim + rot)
+    x = torch.randn(t, 4 + hq + rank + rot + heads + 3, generator=g)
+    offs = (4, 4 + hq, 4 + hq + rank + rot)
+    pos = torch.tensor([0, 1, 17, 4095, 5000, 2], dtype=torch.int64)
+    slots = torch.tensor([4, 0, -1, 7, 2, 5], dtype=torch.int64)
+    wkv = torch.randn(rank, generator=g)
+    freq, mag = lo.ramped_frequencies(rot, 200.0, RAMP)
+    assert mag > 1.05 and freq[0] == 1.0 and freq[2] < 200.0 ** (-4 / 6) / 2.4
+    cache = torch.full((8, row), 9.0).cuda()
+    q, gate = ops.latent_rope_prep(x.cuda(), offs, pos.cuda(), freq.cuda(), mag, wkv.cuda(), eps, slots.cuda(), cache, heads, dim, rot)
+    xq = x[:, 4:4 + hq].double().view(t, heads, dim + rot)
+    want_q = torch.cat([xq[..., :dim], lo.turn_pairs(xq[..., dim:].transpose(0, 1), pos, freq, mag).transpose(0, 1)], -1).reshape(t, hq)
+    assert torch.allclose(q.cpu().double(), want_q, atol=2e-5)
+    assert torch.allclose(gate.cpu().double(), torch.sigmoid(x[:, offs[2]:offs[2] + heads].double()), atol=1e-6)
+    down = x[:, offs[1]:offs[1] + rank + rot].double()
+    want_row = torch.cat([lo.rms(down[:, :rank], eps) * wkv.double(), lo.turn_pairs(down[:, rank:], pos, freq, mag), torch.zeros(t, row - rank - rot).double()], 1)
+    keep = slots >= 0
+    assert torch.allclose(cache.cpu().double()[slots[keep]], want_row[keep], atol=2e-5)
+    assert (cache.cpu()[[1, 3, 6]] == 9.0).all()
+
+
+def _cached(keys, values, n_slots, seed):
+    """Per-sequence keys (T, G, D) and values (T, G, E) put at scattered slots of caches; returns caches and each sequence's slots."""
+    perm = torch.randperm(n_slots, generator=torch.Generator().manual_seed(seed)).tolist()
+    g, d, e = keys[0].shape[1], keys[0].shape[2], values[0].shape[2]
+    kc, vc = torch.zeros(n_slots, g * d), torch.zeros(n_slots, g * e)
+    lists = []
+    for k, v in zip(keys, values):
+        s = [perm.pop() for _ in range(k.shape[0])]
+        kc[s], vc[s] = k.reshape(len(s), -1), v.reshape(len(s), -1)
+        lists.append(s)
+    return kc, vc, lists
+
+
+def _attend(ops, q_rows, lens, totals, lists, kc, vc, fmt, decode, **kw):
+    """ops.softcap_attn for a step that brings the last lens[b] tokens of the first totals[b] of sequence b."""
+    flat = torch.tensor([s for b, l in enumerate(lists) for s in l[:totals[b]]], dtype=torch.int32).cuda()
+    start = torch.tensor(np.concatenate([[0], np.cumsum(totals)[:-1]]), dtype=torch.int64).cuda()
+    kv_len = torch.tensor(totals, dtype=torch.int32).cuda()
+    lay = step_layout(ops, lens, [n - l for n, l in zip(totals, lens)], list(range(len(lens))), decode)
+    return ops.softcap_attn(q_rows.to(fmt).cuda(), kc.to(fmt).cuda(), vc.to(fmt).cuda(), flat, start, kv_len, lay, **kw).float().cpu()
+
+
+def _sink_reference(q, k, v, gate, scale, cap, sink):
+    """Per sequence: every head's read-out with the silent term, times the sigmoid of the head's gate.  (T, heads * vdim)."""
+    heads, kvh = q.shape[1], k.shape[1]
+    pos = torch.arange(q.shape[0])
+    return torch.cat([lo.sink_softmax_readout(q[:, h].double(), k[:, h // (heads // kvh)].double(), v[:, h // (heads // kvh)].double(), pos, pos,
+                                              scale, cap, sink) * torch.sigmoid(gate[:, h:h + 1].double()) for h in range(heads)], -1)
+
+
+@pytest.mark.parametrize("sink", [0.0, None, 1.5])
+@pytest.mark.parametrize("loud", ["first key", "none"])
+def test_attention_with_a_silent_term_and_one_gate_per_head(sink, loud):
+    """Two sequences of unequal length at scattered slots, portions and single tokens, with and without the key split.  With `loud`
+    every query asks loudly for the very first key, hundreds of tokens back; without, the scores are small and the silent term is a
+    large part of the sum, most of all for the first tokens."""
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(7)
+    heads, kvh, dim, vdim, scale, cap = 6, 2, 16, 24, 0.3, 11.0
+    n = [200, 77]
+    q = [torch.randn(t, heads, dim, generator=g) * (1.0 if loud != "none" else 0.3) for t in n]
+    k = [torch.randn(t, kvh, dim, generator=g) for t in n]
+    v = [torch.randn(t, kvh, vdim, generator=g) for t in n]
+    gate = [torch.randn(t, heads + 2, generator=g) for t in n]          # the gates are a slice of wider rows
+    if loud != "none":
+        for b in range(2):
+            for h in range(heads):
+                k0 = k[b][0, h // (heads // kvh)]
+                q[b][:, h] = 5.0 * k0 / k0.norm()
+    want = [_sink_reference(q[b], k[b], v[b], gate[b][:, 2:], scale, cap, sink) for b in range(2)]
+    kc, vc, lists = _cached(k, v, 300, 3)
+    kw = dict(scale=scale, cap=cap, heads=heads, kv_heads=kvh, dim=dim, vdim=vdim, sink_score=sink)
+    for lens, totals, decode in (([200, 77], [200, 77], False), ([3, 70], [131, 77], False), ([1, 1], [66, 65], True), ([1, 1], [200, 2], True),
+                                 ([2, 1], [2, 1], False), ([1, 1], [1, 64], True)):
+        rows = torch.cat([q[b][totals[b] - lens[b]:totals[b]].reshape(lens[b], -1) for b in range(2)])
+        gates = torch.cat([gate[b][totals[b] - lens[b]:totals[b]] for b in range(2)]).cuda()[:, 2:]
+        ref = torch.cat([want[b][totals[b] - lens[b]:totals[b]] for b in range(2)])
+        for split in (1, 4):
+            got = _attend(ops, rows, lens, totals, lists, kc, vc, torch.float32, decode, n_split=split, gate=gates, **kw)
+            close(got, ref, 1e-4, f"lens {lens} of {totals}, split {split}")
+    # the restatement itself depends on the term: without it the weights add up to one
+    if sink is not None and loud == "none":
+        plain = _sink_reference(q[0], k[0], v[0], gate[0][:, 2:], scale, cap, None)
+        assert (plain[:3] - want[0][:3]).abs().max() > 0.05
+
+
+@pytest.mark.parametrize("dim,vdim", [(64, 96), (96, 64), (128, 128)])
+def test_silent_term_and_head_gates_on_the_matrix_cores(dim, vdim):
+    """Steps of many tokens in bfloat16 take the tile kernel: ragged prompts that end in the middle of a key tile and portions that
+    start in the middle of one, a loud first key; against the restatement on the same bfloat16 values and against the vector kernel."""
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(dim)
+    heads, kvh, scale, cap = 4, 2, 0.2, 9.0
+    n = [200, 77, 300, 1]
+    bf = lambda x: x.to(torch.bfloat16).float()
+    q = [bf(torch.randn(t, heads, dim, generator=g) * 0.3) for t in n]
+    k = [bf(torch.randn(t, kvh, dim, generator=g)) for t in n]
+    v = [bf(torch.randn(t, kvh, vdim, generator=g)) for t in n]
+    for b in (0, 2):
+        for h in range(heads):
+            k0 = k[b][0, h // (heads // kvh)]
+            q[b][:, h] = bf(4.0 * k0 / k0.norm())
+    gate = [bf(torch.randn(t, heads, generator=g)) for t in n]
+    want = [_sink_reference(q[b], k[b], v[b], gate[b], scale, cap, 0.0) for b in range(len(n))]
+    kc, vc, lists = _cached(k, v, 700, 5)
+    kw = dict(scale=scale, cap=cap, heads=heads, kv_heads=kvh, dim=dim, vdim=vdim, sink_score=0.0, n_split=1)
+    for lens, totals in ((n, n), ([70, 3, 130, 1], [200, 77, 300, 1]), ([129, 77, 1, 1], [130, 77, 65, 1])):
+        rows = torch.cat([q[b][totals[b] - lens[b]:totals[b]].reshape(lens[b], -1) for b in range(len(n))])
+        gates = torch.cat([gate[b][totals[b] - lens[b]:totals[b]] for b in range(len(n))]).to(torch.bfloat16).cuda()
+        ref = torch.cat([want[b][totals[b] - lens[b]:totals[b]] for b in range(len(n))])
+        tile = _attend(ops, rows, lens, totals, lists, kc, vc, torch.bfloat16, False, gate=gates, matrix_cores=True, **kw)
+        vec = _attend(ops, rows, lens, totals, lists, kc, vc, torch.bfloat16, False, gate=gates, matrix_cores=False, **kw)
+        for got, what in ((tile, "matrix cores"), (vec, "vector units")):
+            err = ((got.double() - ref).abs() / (ref.abs() + 0.05 * ref.std())).max().item()
+            assert err < 8e-3, f"{what}, lens {lens} of {totals}: {err:.2e}"
+
+
+def _walk(full, cuts, slot, order, run):
+    """Sequences `full` (id -> rows) cut into steps (`cuts`: id -> sizes), `order` naming the live ids of every step; run(x, lens,
+    pos0, slots, decode) -> rows.  Returns id -> all rows."""
+    at = {i: 0 for i in full}
+    got = {i: [] for i in full}
+    for live in order:
+        live = [i for i in live if at[i] < len(full[i]) and cuts[i]]
+        if not live:
+            continue
+        lens = [cuts[i].pop(0) for i in live]
+        x = torch.cat([full[i][at[i]:at[i] + n] for i, n in zip(live, lens)])
+        decode = all(n == 1 for n in lens) and all(at[i] > 0 for i in live)
+        out = run(x, lens, [at[i] for i in live], [slot[i] for i in live], decode)
+        a = 0
+        for i, n in zip(live, lens):
+            got[i].append(out[a:a + n])
+            a += n
+            at[i] += n
+    assert all(at[i] == len(full[i]) for i in full)
+    return {i: torch.cat(r) for i, r in got.items()}
+
+
+ORDER = [[0, 1]] * 4 + [[0]] * 10 + [[1]] * 5 + [[2, 1]] * 5 + [[2]] * 4
+
+
+@pytest.mark.parametrize("taps,channels", [(1, 7), (2, 33), (4, 24), (5, 300)])
+def test_short_convolution_with_a_bias_over_cuts_and_reused_slots(taps, channels):
+    """Portions shorter than the taps, single tokens, a sequence that takes over a used slot and must see zeros before its start."""
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(taps)
+    full = {0: torch.randn(130, channels + 3, generator=g), 1: torch.randn(17, channels + 3, generator=g), 2: torch.randn(9, channels + 3, generator=g)}
+    w, b = torch.randn(channels, taps, generator=g), torch.randn(channels, generator=g)
+    want = {i: lo.causal_conv(x[:, 3:].double(), w.double(), b.double()) for i, x in full.items()}
+    state = torch.full((3, taps - 1, channels), 7.0).cuda() if taps > 1 else None
+    cuts = {0: cuts_of(130, [1, 2, 9, 8, 1, 1, 130]), 1: cuts_of(17, [5, 1, 1, 2, 17]), 2: cuts_of(9, [2, 1, 6])}
+
+    def run(x, lens, pos0, slots, decode):
+        return ops.short_conv(x.cuda()[:, 3:], w.t().contiguous().cuda(), state, step_layout(ops, lens, pos0, slots, decode), bias=b.cuda()).cpu()
+    got = _walk(full, cuts, {0: 2, 1: 0, 2: 2}, ORDER, run)
+    for i in full:
+        close(got[i], want[i], 1e-5, f"sequence {i}")
+
+
+@pytest.mark.parametrize("width,blocks", [(24, 3), (7, 1), (66, 2), (300, 300)])
+def test_gated_recurrence_over_cuts_and_reused_slots(width, blocks):
+    """Two sequences in slots that are not in order, cut into steps of 1, 2 and more tokens; a third sequence later takes over a
+    used slot and must start from zero.  Channels whose decay is close to one keep the first token for hundreds of steps."""
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(width)
+    bw = width // blocks
+    # rows: y | u | per block [recurrence gate | input gate]
+    full = {0: torch.randn(330, 4 * width, generator=g), 1: torch.randn(17, 4 * width, generator=g), 2: torch.randn(9, 4 * width, generator=g)}
+    lam = torch.randn(width, generator=g) * 3.0 - 6.0                       # decays between about 0.5 and 0.99999 a step
+    bias = torch.randn(2, width, generator=g)
+
+    def ref(x):
+        x = x.double()
+        gates = x[:, 2 * width:].view(-1, blocks, 2 * bw)
+        r = gates[..., :bw].reshape(-1, width) + bias[0].double()
+        i = gates[..., bw:].reshape(-1, width) + bias[1].double()
+        return lo.gated_recurrence(x[:, width:2 * width], r, i, lam.double()) * lo.gelu_tanh(x[:, :width])
+    want = {i: ref(x) for i, x in full.items()}
+    rate = (8.0 * torch.nn.functional.softplus(lam.double())).float().cuda()
+    state = torch.full((3, width), 7.0).cuda()
+    cuts = {0: cuts_of(330, [1, 2, 9, 8, 1, 1, 200, 1, 1, 130]), 1: cuts_of(17, [5, 1, 1, 2, 17]), 2: cuts_of(9, [2, 1, 6])}
+
+    def run(x, lens, pos0, slots, decode):
+        x = x.cuda()
+        gates = x[:, 2 * width:].reshape(-1, blocks, 2 * bw).transpose(0, 1).contiguous()
+        return ops.rglru_scan(x[:, :width], x[:, width:2 * width], gates, bias.cuda(), rate, state, step_layout(ops, lens, pos0, slots, decode)).cpu()
+    got = _walk(full, cuts, {0: 2, 1: 0, 2: 2}, ORDER, run)
+    for i in full:
+        close(got[i], want[i], 1e-4, f"sequence {i}")
+    # the state left behind is the last S itself
+    x = full[2].double()
+    gates = x[:, 2 * width:].view(-1, blocks, 2 * bw)
+    last = lo.gated_recurrence(x[:, width:2 * width], gates[..., :bw].reshape(-1, width) + bias[0].double(),
+                               gates[..., bw:].reshape(-1, width) + bias[1].double(), lam.double())[-1]
+    close(state[2].cpu(), last, 1e-4, "state of the last sequence in slot 2")
+    # the first token still counts at the end of the long sequence, in the slowest channels
+    slow = lam < -8.0
+    if slow.any():
+        assert ((ref(full[0][1:])[-1] - want[0][-1]).abs()[slow] / (want[0][-1].abs()[slow] + 1e-3)).max() > 1e-3
+
+
+@pytest.mark.parametrize("experts,top,groups,keep", [(6, 3, 3, 2), (16, 4, 4, 3), (4, 1, 0, 0), (8, 3, 4, 4), (12, 6, 2, 1), (5, 5, 0, 0), (9, 2, 9, 2), (6, 2, 3, 2)])
+def test_softmax_router_with_groups(experts, top, groups, keep):
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(experts)
+    z = torch.randn(300, experts, generator=g) * 2.0
+    router = {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep} if groups else None}
+    ids, wts = lo.route_logits(z.double(), router)
+    got_i, got_w = ops.moe_route_softmax(z.cuda(), top, groups, keep, 1e-20)
+    order = got_i.cpu().long().sort(1)
+    want_order = ids.sort(1)
+    assert torch.equal(order.values, want_order.values)
+    assert torch.allclose(got_w.cpu().double().gather(1, order.indices), wts.gather(1, want_order.indices), atol=1e-6)
+    assert torch.allclose(got_w.sum(1).cpu(), torch.ones(300), atol=1e-5)
+    if groups and keep < min(top, groups):       # the groups matter: without them other experts are chosen somewhere
+        free, _ = lo.route_logits(z.double(), {"experts": experts, "top": top})
+        assert not torch.equal(free.sort(1).values, want_order.values)
+
+
+@pytest.mark.parametrize("experts,top,groups,keep", [(6, 3, 3, 2), (3, 3, 0, 0), (4, 1, 2, 1)])
+def test_grouped_experts_by_rows_and_by_expert_order(experts, top, groups, keep):
+    from nano_vllm_x_amd.layers.moe import GroupedSoftmaxMoE
+    g = torch.Generator().manual_seed(top)
+    width, ff, t, limit = 40, 24, 50, 0.9
+    p = {f"e{j}.{s}": torch.randn((ff, width) if s != "down" else (width, ff), generator=g) * 0.3 for j in range(experts) for s in ("gate", "up", "down")}
+    p["router"] = torch.randn(experts, width, generator=g) * 0.5
+    moe = GroupedSoftmaxMoE(width, experts, top, ff, limit, 1.702, 1.0, groups=groups or None, keep=keep or None).float().cuda()
+    with torch.no_grad():
+        for j in range(experts):
+            moe.w_gu[j, :ff], moe.w_gu[j, ff:], moe.w_d[j] = p[f"e{j}.gate"].cuda(), p[f"e{j}.up"].cuda(), p[f"e{j}.down"].cuda()
+        moe.router.copy_(p["router"])
+    h = torch.randn(t, width, generator=g)
+    mlp = {"expert": {"ff": ff, "limit": limit}, "router": {"experts": experts, "top": top, "groups": {"count": groups, "keep": keep} if groups else None}}
+    want = lo.moe_ff(h.double(), {k: v.double() for k, v in p.items()}, "", mlp)
+    with torch.inference_mode():
+        close(moe(h.cuda(), decode_step=False).cpu(), want, 1e-4, "expert order")
+        close(moe(h.cuda(), decode_step=True).cpu(), want, 1e-4, "rows")
+        close(moe(h[:3].cuda()).cpu(), want[:3], 1e-4, "few tokens")
+
+
+# ---- one mixer at a time -------------------------------------------------------------------------------------------------
+def _att(mlp=None, **changes):
+    return {"type": "attention", "mixer": dict(ATT["mixer"], **changes), "mlp": mlp}
+
+
+ONE = {
+    "attention": ([_att()], 3),
+    "attention, one stream with weights": ([_att()], 1),
+    "attention, a plain residual sum": ([_att(DENSE)], None),
+    "attention, whole head rotated, no cap, no scaling": ([_att(dim=8, vdim=8, softcap=None, rot={"dims": 8, "base": 77.0})], 2),
+    "attention, one head of one key": ([_att(heads=1, kv_heads=1, dim=2, vdim=1, rot={"dims": 2, "base": 10.0})], 2),
+    "attention, borrowed keys": ([REC, ATT, borrowing(ATT, 1, None), borrowing(ATT, 1, DENSE, heads=2, scale=0.5)], 3),
+    "latent attention": ([dict(LAT, mlp=None)], 3),
+    "latent attention, nothing unrotated in common sizes": ([{"type": "latent_attention", "mlp": None, "mixer": {
+        "heads": 2, "dim": 3, "rot_dim": 2, "vdim": 5, "kv_rank": 31, "scale": 0.4, "rot": {"dims": 2, "base": 50.0}}}], 2),
+    "recurrence": ([dict(REC, mlp=None)], 3),
+    "recurrence, one tap, one block": ([{"type": "rglru", "mixer": {"width": 10, "blocks": 1, "conv": 1}, "mlp": None}], 2),
+    "recurrence, blocks of one channel": ([{"type": "rglru", "mixer": {"width": 6, "blocks": 6, "conv": 2}, "mlp": None}], 4),
+    "dense feed-forward": ([dict(REC, mlp=DENSE)], 3),
+    "experts in groups": ([dict(REC, mlp=MOE)], 3),
+    "experts, all of all": ([dict(REC, mlp={"kind": "moe", "expert": {"ff": 8, "limit": 0.5}, "router": {"experts": 3, "top": 3}})], 3),
+    "experts, every group kept": ([dict(REC, mlp={"kind": "moe", "expert": {"ff": 8, "limit": 3.0},
+                                                  "router": {"experts": 6, "top": 2, "groups": {"count": 2, "keep": 2}}})], 3),
+}
+
+
+@pytest.mark.parametrize("name", list(ONE))
+def test_each_mixer_alone_whole_cut_and_token_by_token(tmp_path, name):
+    layers, streams = ONE[name]
+    cfg = make_cfg(layers, streams=streams)
+    w = weights_of(cfg, 1)
+    eng = make_engine(model_dir(tmp_path, cfg, w), pool=256)
+    toks = tokens(70, cfg["vocab"], 3)
+    want = forward(cfg, w, toks)
+    close(replay(eng, {"a": toks}, [[("a", 70)]])["a"], want, F32_TOL, "whole")
+    close(replay(eng, {"b": toks}, [[("b", n)] for n in cuts_of(70, [2, 7, 1, 9, 3, 8, 16])])["b"], want, F32_TOL, "cut")
+    close(replay(eng, {"c": toks}, [[("c", 1)]] * 70)["c"], want, F32_TOL, "token by token")
+    eng.shutdown()
+
+
+def test_residual_after_every_layer(tmp_path):
+    """The sum of the streams after each layer, as the model can record it, against the restatement's."""
+    cfg = make_cfg([ATT, LAT, REC, borrowing(ATT, 0, MOE)])
+    w = weights_of(cfg, 5)
+    eng = make_engine(model_dir(tmp_path, cfg, w), pool=128)
+    toks = tokens(23, cfg["vocab"], 1)
+    sums = []
+    lo.forward(cfg, w, toks, sums)
+    model = eng.model_runner.model
+    model.layer_streams = []
+    replay(eng, {"a": toks}, [[("a", 23)]])
+    got, model.layer_streams = model.layer_streams, None
+    assert len(got) == len(sums) == 4
+    for i, (a, b) in enumerate(zip(got, sums)):
+        close(a.float().cpu(), b, 5e-5, f"after layer {i}")
+    eng.shutdown()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_that_fit_no_vector_width(tmp_path, dtype):
+    """A width, head sizes, ranks, feed-forward sizes and a vocabulary that are multiples of nothing useful (no 16-byte rows
+    anywhere), three query heads on one key/value head, five streams, experts in the first layer and none in the last."""
+    odd = [{"type": "attention", "mixer": {"heads": 3, "kv_heads": 1, "dim": 10, "vdim": 6, "scale": 0.3, "softcap": 2.5, "rot": {"dims": 6, "base": 41.0}},
+            "mlp": {"kind": "moe", "expert": {"ff": 9, "limit": 1.1}, "router": {"experts": 9, "top": 3, "groups": {"count": 3, "keep": 1}}}},
+           {"type": "rglru", "mixer": {"width": 15, "blocks": 5, "conv": 3}, "mlp": {"kind": "dense", "ff": 11}},
+           {"type": "latent_attention", "mixer": {"heads": 5, "dim": 7, "rot_dim": 4, "vdim": 3, "kv_rank": 13, "scale": 0.2,
+                                                  "rot": {"dims": 4, "base": 900.0, "scaling": {"factor": 8.0, "original": 16, "fast": 2.0, "slow": 0.25}}},
+            "mlp": {"kind": "dense", "ff": 7}},
+           borrowing({"mixer": {"heads": 1, "kv_heads": 1, "dim": 10, "vdim": 6, "scale": 1.0, "rot": {"dims": 6, "base": 41.0}}}, 0, None)]
+    cfg = make_cfg(odd, width=50, vocab=37, emb=1.0, streams=5)
+    cfg.pop("embedding")
+    w = weights_of(cfg, 4)
+    eng = make_engine(model_dir(tmp_path, cfg, w), dtype=dtype, pool=256)
+    toks = tokens(45, 37, 8)
+    want = forward(cfg, w, toks)
+    got = replay(eng, {"a": toks}, [[("a", 33)], [("a", 2)]] + [[("a", 1)]] * 10)["a"]
+    if dtype == "float32":
+        close(got, want, F32_TOL, "float32")
+        close(replay(eng, {"b": toks}, [[("b", 45)]])["b"], want, F32_TOL, "whole")
+    else:
+        err = (got.double() - want).abs().amax(dim=1) / want.std()
+        assert err.median() < 0.08 and err.max() < 0.4, (err.median().item(), err.max().item())
+    eng.shutdown()
+
+
+def test_first_tokens_and_page_borders_in_prompts_and_decoding(tmp_path):
+    """Prompts of 1, 2, 63, 64, 65, 128, 129 tokens; pages of 64 and key tiles crossed token by token and by portions that start or
+    end at them; sharpened scores."""
+    cfg = make_cfg([ATT, LAT, REC, borrowing(ATT, 0)])
+    w = sharpen(weights_of(cfg, 12))
+    eng = make_engine(model_dir(tmp_path, cfg, w), pool=1024)
+    toks = tokens(200, cfg["vocab"], 6)
+    want = forward(cfg, w, toks)
+    for n in (1, 2, 3, 63, 64, 65, 128, 129):
+        close(replay(eng, {f"p{n}": toks[:n]}, [[(f"p{n}", n)]])[f"p{n}"], want[:n], F32_TOL, f"prompt of {n}")
+    sched = [[("a", 1)]] * 3 + [[("a", 59)]] + [[("a", 1)]] * 4 + [[("a", 2)], [("a", 58)], [("a", 2)], [("a", 2)]] + [[("a", 1)]] * 5 + \
+            [[("a", 64)]] + [[("a", 1)]]
+    assert sum(n for step in sched for _, n in step) == 200
+    close(replay(eng, {"a": toks}, sched)["a"], want, F32_TOL, "borders crossed token by token")
+    eng.shutdown()
+
+
+# ---- the whole stack ------------------------------------------------------------------------------------------------------
+def test_batches_of_unequal_requests_in_a_small_pool(tmp_path):
+    """Four live requests at most in a pool smaller than the sum of all: portions beside single tokens, a request that
+    pauses for some steps, token slots and state slots that change hands (six requests, four state slots)."""
+    cfg = make_cfg([REC, ATT, LAT, borrowing(ATT, 1), REC])
+    w = weights_of(cfg, 2)
+    eng = make_engine(model_dir(tmp_path, cfg, w), pool=160, max_bs=4)
+    req = {f"r{k}": tokens(n, cfg["vocab"], 30 + k) for k, n in enumerate([70, 41, 1, 23, 55, 38])}
+    want = {i: forward(cfg, w, t) for i, t in req.items()}
+    sched = [[("r0", 16), ("r1", 2)], [("r0", 1), ("r1", 30), ("r2", 1)], [("r0", 40), ("r3", 3)], [("r1", 1), ("r3", 1)],
+             [("r0", 1), ("r1", 1), ("r3", 17)], [("r0", 12), ("r1", 7), ("r3", 2)],          # r0, r1, r3 done: 134 slots come back
+             [("r4", 2), ("r5", 30)], [("r4", 50), ("r5", 1)], [("r4", 1), ("r5", 1)], [("r4", 2), ("r5", 6)]]
+    got = replay(eng, req, sched)
+    for i in req:
+        close(got[i], want[i], F32_TOL, i)
+    assert eng.scheduler.state_slots.num_free() == 4
+    eng.shutdown()
+
+
+def test_far_tokens_and_old_state_count(tmp_path):
+    """Sharpened scores over 330 tokens, decoded one by one at the end: the first token must still be seen, through the attention
+    layers (all earlier keys count) and through the slow channels of the recurrence."""
+    cfg = make_cfg([REC, ATT, LAT, borrowing(ATT, 1)])
+    w = sharpen(weights_of(cfg, 7))
+    w["l0.mix.lam"] = (w["l0.mix.lam"] - 6.0).to(torch.bfloat16).float()          # slow decays: the state remembers hundreds of tokens
+    eng = make_engine(model_dir(tmp_path, cfg, w), pool=512)
+    toks = tokens(330, cfg["vocab"], 2)
+    want = forward(cfg, w, toks)
+    got = replay(eng, {"a": toks}, [[("a", 255)], [("a", 1)], [("a", 1)], [("a", 2)], [("a", 30)]] + [[("a", 1)]] * 41)["a"]
+    close(got, want, F32_TOL, "sharpened")
+    other = forward(cfg, w, toks[1:])
+    assert (other[-1] - want[-1]).abs().max() > 8 * F32_TOL * want.std()
+    eng.shutdown()
+
+
+def test_bfloat16_stays_within_rounding(tmp_path):
+    cfg = make_cfg([ATT, LAT, REC, borrowing(ATT, 0)])
+    toks = tokens(90, cfg["vocab"], 4)
+    want = forward(cfg, weights_of(cfg, 2), toks)
+    eng = make_engine(model_dir(tmp_path, cfg), dtype="bfloat16", seed=2)
+    got = replay(eng, {"a": toks}, [[("a", 50)], [("a", 2)]] + [[("a", 1)]] * 38)["a"]
+    err = (got.double() - want).abs().amax(dim=1) / want.std()
+    assert err.median() < 0.08 and err.max() < 0.4, (err.median().item(), err.max().item())
+    eng.shutdown()
+
+
+def test_bfloat16_with_heads_for_the_matrix_cores(tmp_path):
+    """Head sizes the tile kernels are built for (keys 64, values 128; a latent row of 96), prompts long enough to take them, in
+    bfloat16: whole prompts against portions and single tokens, and both against the restatement within rounding."""
+    att = {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 64, "vdim": 128, "scale": 0.125, "softcap": 20.0,
+                                          "rot": {"dims": 32, "base": 1e4, "scaling": {"factor": 2.0, "low": 1.0, "high": 4.0, "original": 32}}}, "mlp": DENSE}
+    lat = {"type": "latent_attention", "mixer": {"heads": 4, "dim": 32, "rot_dim": 16, "vdim": 48, "kv_rank": 80, "scale": 0.14,
+                                                 "rot": {"dims": 16, "base": 1e4, "scaling": RAMP}}, "mlp": MOE}
+    cfg = make_cfg([att, lat, borrowing(att, 0)], width=128, vocab=97, emb=8.0)
+    w = weights_of(cfg, 3)
+    eng = make_engine(model_dir(tmp_path, cfg, w), dtype="bfloat16", pool=1024)
+    toks = tokens(300, 97, 9)
+    want = forward(cfg, w, toks)
+    whole = replay(eng, {"a": toks}, [[("a", 300)]])["a"]
+    cut = replay(eng, {"b": toks}, [[("b", 130)], [("b", 100)], [("b", 2)], [("b", 63)]] + [[("b", 1)]] * 5)["b"]
+    for got, what in ((whole, "whole"), (cut, "cut")):
+        err = (got.double() - want).abs().amax(dim=1) / want.std()
+        assert err.median() < 0.08 and err.max() < 0.4, (what, err.median().item(), err.max().item())
+    eng.shutdown()
+
+
+def test_checkpoint_with_a_missing_or_misshapen_tensor_is_refused(tmp_path):
+    cfg = make_cfg([ATT, REC, LAT])
+    w = weights_of(cfg, 0)
+    for gone in ("l0.hc2.mix", "l1.mix.ri.b", "l2.mix.dkv.norm", "l0.mix.o.b"):
+        bad = dict(w)
+        del bad[gone]
+        with pytest.raises(KeyError):
+            make_engine(model_dir(tmp_path, cfg, bad, name="missing_" + gone.replace(".", "_")))
+    bad = dict(w)
+    bad["l1.mix.conv"] = torch.zeros(24, 3)
+    with pytest.raises(ValueError):
+        make_engine(model_dir(tmp_path, cfg, bad, name="shape"))
+    bad = dict(w)
+    bad["l1.mix.k"] = torch.zeros(24, 40)
+    with pytest.raises(KeyError):
+        make_engine(model_dir(tmp_path, cfg, bad, name="extra"))
+
+
+# ---- generation: the scheduler's own choices ---------------------------------------------------------------------------
+def oracle_greedy(w, cfg, prompt, n_new):
+    return greedy(lambda t: forward(cfg, w, t), prompt, n_new)
+
+
+@pytest.mark.parametrize("chunked", [False, True], ids=["whole prompts", "chunked prefill"])
+def test_greedy_generation_through_the_engine(tmp_path, chunked):
+    """Prompts of unequal length admitted together, decoded as one batch; more requests than state slots, so the later ones wait
+    for a slot that an earlier one gives back; with chunked prefill the prompts are computed in portions of seven tokens.  Long
+    decoding (70 tokens, across a page of 64) for one of them."""
+    from nano_vllm_x_amd.core.common import SamplingParams
+    cfg = make_cfg([REC, ATT, LAT, borrowing(ATT, 1)])
+    kw = dict(max_prefill_tokens=7, chunked_prefill=True) if chunked else {}
+    eng = make_engine(model_dir(tmp_path, cfg), pool=400, max_bs=3, seed=9, **kw)
+    w = weights_of(cfg, 9)
+    prompts = {f"r{k}": tokens(n, cfg["vocab"], 20 + k) for k, n in enumerate([5, 19, 1, 12, 9])}
+    new = {"r0": 70, "r1": 5, "r2": 8, "r3": 4, "r4": 6}
+    for i, p in prompts.items():
+        eng.add_sequence(i, list(p), SamplingParams(temperature=0.0, ignore_eos=True, max_new_tokens=new[i]))
+    out = {i: [] for i in prompts}
+    steps = 0
+    while eng.has_unfinished_sequences():
+        for o in eng.step():
+            out[o.seq_id].append(o.new_token_id)
+        steps += 1
+        assert steps < 600
+    for i, p in prompts.items():
+        assert out[i] == oracle_greedy(w, cfg, p, new[i]), i
+    assert eng.scheduler.state_slots.num_free() == 3
+    eng.shutdown()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_decode_steps_replay_a_captured_graph(tmp_path, dtype):
+    """With graphs on, every decode step replays the graph of its batch size, with prefill steps of later requests (eager work on
+    the same cache and state) between the replays; batch sizes change as requests end.  float32: the tokens are the
+    restatement's; bfloat16: the graph's tokens are those of eager steps (same kernels, same order)."""
+    from nano_vllm_x_amd.core.common import SamplingParams
+    from nano_vllm_x_amd.core.engine import Engine
+    cfg = make_cfg([REC, ATT, LAT, borrowing(ATT, 1, DENSE)])
+    path = model_dir(tmp_path, cfg)
+    prompts = {f"r{k}": tokens(n, cfg["vocab"], 40 + k) for k, n in enumerate([9, 26, 2, 17, 5])}
+    new = {"r0": 20, "r1": 5, "r2": 11, "r3": 3, "r4": 7}
+
+    def run(eager):
+        eng = Engine(model=path, gpu_memory_utilization=0.5, max_bs=3, enforce_eager=eager, context_len=128, kv_cache_size=300,
+                     dtype=dtype, seed=5)
+        for i, p in prompts.items():
+            eng.add_sequence(i, list(p), SamplingParams(temperature=0.0, ignore_eos=True, max_new_tokens=new[i]))
+        out = {i: [] for i in prompts}
+        while eng.has_unfinished_sequences():
+            for o in eng.step():
+                out[o.seq_id].append(o.new_token_id)
+        stats = dict(eng.model_runner.stats)
+        eng.shutdown()
+        return out, stats
+
+    got, stats = run(False)
+    assert stats["graph_steps"] > 15 and stats["eager_decode_steps"] == 0
+    if dtype == "float32":
+        w = weights_of(cfg, 5)
+        for i, p in prompts.items():
+            assert got[i] == oracle_greedy(w, cfg, p, new[i]), i
+    else:
+        assert got == run(True)[0]
+
+
+def test_generate_entry_point(tmp_path):
+    from nano_vllm_x_amd import LLM, SamplingParams
+    cfg = make_cfg([ATT, REC, LAT], vocab=300)
+    llm = LLM(model_dir(tmp_path, cfg), gpu_memory_utilization=0.5, max_bs=2, enforce_eager=True, context_len=256, kv_cache_size=256,
+              dtype="float32", seed=4)
+    prompt = tokens(11, 300, 1)
+
+    async def run():
+        ids = []
+        async for o in llm.generate(list(prompt), SamplingParams(temperature=0.0, ignore_eos=True, max_new_tokens=5, eos_token_id=0)):
+            ids.append(o.token_id)
+        return ids
+
+    assert asyncio.run(run()) == oracle_greedy(weights_of(cfg, 4), cfg, prompt, 5)
+    llm.shutdown()
+
+
+def test_preempted_sequence_starts_again_from_an_empty_state(tmp_path):
+    from nano_vllm_x_amd.core.common import SamplingParams
+    cfg = make_cfg([REC, ATT, LAT])
+    eng = make_engine(model_dir(tmp_path, cfg), pool=64, max_bs=2, seed=6)
+    w = weights_of(cfg, 6)
+    prompts = {"a": tokens(20, cfg["vocab"], 1), "b": tokens(25, cfg["vocab"], 2)}
+    for i, p in prompts.items():
+        eng.add_sequence(i, list(p), SamplingParams(temperature=0.0, ignore_eos=True, max_new_tokens=14))
+    out = {i: [] for i in prompts}
+    while eng.has_unfinished_sequences():       # 45 + 2 * 14 tokens do not fit 64 slots: the younger sequence is preempted
+        for o in eng.step():
+            out[o.seq_id].append(o.new_token_id)
+    for i, p in prompts.items():
+        assert out[i] == oracle_greedy(w, cfg, p, 14), i
+    eng.shutdown()
+
+
+def test_command_line_generates_what_the_restatement_does(tmp_path):
+    import subprocess
+    import sys
+    cfg = make_cfg([ATT, REC, LAT], vocab=90)
+    path = model_dir(tmp_path, cfg)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-m", "nano_vllm_x_amd", "--model", path, "--prompt-ids", "5,17,3,44", "--prompt-ids", "8",
+                          "--max-new-tokens", "6", "--dtype", "float32", "--kv-cache-size", "128", "--context-len", "64", "--max-bs", "2",
+                          "--seed", "3"], cwd=root, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr[-2000:]
+    lines = [json.loads(x) for x in out.stdout.splitlines() if x.startswith("{")]
+    w = weights_of(cfg, 3)
+    assert [x["prompt"] for x in lines] == [[5, 17, 3, 44], [8]]
+    for x in lines:
+        assert x["generated_ids"] == oracle_greedy(w, cfg, x["prompt"], 6)
+
+
+def test_trace_runner_replays_steps_from_standard_input(tmp_path):
+    """bin/trace_run on a model directory: two requests, portions beside single tokens, one request ended and its id used again;
+    the logits it writes are the restatement's."""
+    import subprocess
+    cfg = make_cfg([REC, ATT, LAT, borrowing(ATT, 1)], vocab=80)
+    w = weights_of(cfg, 11)
+    path = model_dir(tmp_path, cfg, w)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    a, b = tokens(30, 80, 1), tokens(12, 80, 2)
+    steps = [{"step": 0, "entries": [{"id": "a", "tokens": a[:9], "want": [0, 8]}, {"id": "b", "tokens": b[:1], "want": [0]}], "end": []},
+             {"step": 1, "entries": [{"id": "a", "tokens": a[9:29], "want": []}, {"id": "b", "tokens": b[1:], "want": [10]}], "end": ["b"]},
+             {"step": 2, "entries": [{"id": "a", "tokens": a[29:], "want": [0]}, {"id": "b", "tokens": a[:5], "want": [4]}], "end": ["a", "b"]}]
+    out_dir = tmp_path / "out"
+    r = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", path, "--dtype", "float32", "--out", str(out_dir), "--max-tokens", "128"],
+                       input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=600, cwd=root)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert [x for x in r.stdout.splitlines() if x.startswith("done")] == ["done 0", "done 1", "done 2"]
+    la, lb = forward(cfg, w, a), forward(cfg, w, b)
+    got = [torch.from_numpy(np.fromfile(out_dir / f"{k}.f32", dtype="<f4").reshape(-1, 80).copy()) for k in range(3)]
+    close(got[0], torch.stack([la[0], la[8], lb[0]]), F32_TOL, "step 0")
+    close(got[1], lb[11:12], F32_TOL, "step 1")
+    close(got[2], torch.stack([la[29], la[4]]), F32_TOL, "step 2")

@@ -1,0 +1,181 @@
+"""Host side of the Ladusun family, without a device: configuration, registry, checkpoint names and where their tensors land in
+the fused parameters, frequency tables, and properties of the restatement that the GPU tests lean on."""
+import json
+import math
+
+import pytest
+import torch
+
+from oracle import ladusun_oracle as lo
+
+BANDS = {"factor": 3.0, "low": 0.5, "high": 4.0, "original": 64}
+RAMP = {"factor": 2.5, "original": 48, "fast": 4.0, "slow": 0.5}
+LAYERS = [{"type": "rglru", "mixer": {"width": 20, "blocks": 2, "conv": 3}, "mlp": None},
+          {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 10, "vdim": 6, "scale": 0.3, "softcap": 12.0,
+                                          "rot": {"dims": 8, "base": 300.0, "scaling": BANDS}}, "mlp": {"kind": "dense", "ff": 22}},
+          {"type": "latent_attention", "mixer": {"heads": 3, "dim": 8, "rot_dim": 6, "vdim": 5, "kv_rank": 7, "scale": 0.2,
+                                                 "rot": {"dims": 6, "base": 200.0, "scaling": RAMP}},
+           "mlp": {"kind": "moe", "expert": {"ff": 18, "limit": 1.5}, "router": {"experts": 6, "top": 2, "groups": {"count": 3, "keep": 1}}}},
+          {"type": "attention", "mixer": {"heads": 2, "kv_heads": 2, "dim": 10, "vdim": 6, "scale": 0.1, "kv_from": 1,
+                                          "rot": {"dims": 8, "base": 300.0, "scaling": BANDS}},
+           "mlp": {"kind": "moe", "expert": {"ff": 4, "limit": 9.0}, "router": {"experts": 3, "top": 1}}}]
+CFG = {"architecture": "Ladusun", "vocab": 53, "width": 36, "norm": {"eps": 1e-6}, "embedding": {"scale": 4.0}, "streams": 2, "layers": LAYERS}
+
+
+def test_registry_reads_the_configuration_from_a_directory(tmp_path):
+    from nano_vllm_x_amd.ladusun import LadusunConfig, LadusunForCausalLM
+    from nano_vllm_x_amd.registry import load_config, model_class_of
+    (tmp_path / "config.json").write_text(json.dumps(CFG))
+    cfg = load_config(str(tmp_path))
+    assert isinstance(cfg, LadusunConfig) and model_class_of(cfg) is LadusunForCausalLM and LadusunForCausalLM.family == "seq_state"
+    assert (cfg.vocab_size, cfg.width, cfg.hidden_size, cfg.eps, cfg.embedding_scale, cfg.streams, cfg.n_streams) == (53, 36, 36, 1e-6, 4.0, 2, 2)
+    assert [l["type"] for l in cfg.layers] == ["rglru", "attention", "latent_attention", "attention"] and cfg.layers[0]["mlp"] is None
+    att = cfg.layers[1]["mixer"]
+    assert att["softcap"] == 12.0 and att["rot"] == {"dims": 8, "base": 300.0, "interleaved": True, "scaling": BANDS}
+    assert cfg.layers[3]["mixer"]["kv_from"] == 1 and cfg.layers[3]["mixer"]["softcap"] is None
+    assert cfg.layers[2]["mixer"]["rot"]["dims"] == 6 and cfg.layers[2]["mlp"]["router"]["groups"] == {"count": 3, "keep": 1}
+    assert cfg.layers[3]["mlp"]["router"]["groups"] is None
+    again = LadusunConfig.from_dict(json.loads(json.dumps(cfg.to_dict())))
+    assert again.layers == cfg.layers and again.eps == cfg.eps and again.streams == 2
+    plain = LadusunConfig.from_dict({k: v for k, v in CFG.items() if k not in ("streams", "embedding")})
+    assert plain.streams is None and plain.n_streams == 1 and plain.embedding_scale == 1.0
+    with pytest.raises(ValueError):
+        LadusunConfig.from_dict({**CFG, "layers": [{"type": "conv", "mixer": {}, "mlp": None}]})
+    with pytest.raises(ValueError):      # keys borrowed from a later layer, from one that borrows, or from a layer of another kind
+        LadusunConfig.from_dict({**CFG, "layers": [LAYERS[3], LAYERS[1]]})
+    with pytest.raises(ValueError):
+        LadusunConfig.from_dict({**CFG, "layers": LAYERS + [{**LAYERS[3], "mixer": {**LAYERS[3]["mixer"], "kv_from": 3}}]})
+    with pytest.raises(ValueError):
+        LadusunConfig.from_dict({**CFG, "layers": LAYERS[:3] + [{**LAYERS[3], "mixer": {**LAYERS[3]["mixer"], "kv_from": 0}}]})
+    with pytest.raises(ValueError):      # other key/value sizes than the lender's
+        LadusunConfig.from_dict({**CFG, "layers": LAYERS[:3] + [{**LAYERS[3], "mixer": {**LAYERS[3]["mixer"], "vdim": 8}}]})
+    with pytest.raises(ValueError):
+        LadusunConfig.from_dict({**CFG, "layers": [{**LAYERS[1], "mlp": {"kind": "glu", "ff": 4}}]})
+
+
+def test_checkpoint_tensors_land_in_the_fused_parameters():
+    from nano_vllm_x_amd.ladusun import LadusunConfig, LadusunForCausalLM, checkpoint_shapes, random_checkpoint
+    cfg = LadusunConfig.from_dict(CFG)
+    w = dict(random_checkpoint(cfg, 3))
+    assert {k: tuple(v.shape) for k, v in w.items()} == checkpoint_shapes(cfg)
+    assert "l0.norm2" not in w and "l0.hc2.in" not in w and "l3.mix.k" not in w and "l3.mix.v.b" not in w and "l3.mix.q.b" in w and "l2.mlp.e5.down" in w
+    assert w["l1.hc1.mix"].shape == (2, 2) and w["l1.mix.g"].shape == (4, 36) and w["l2.mix.dkv"].shape == (13, 36) and w["l0.mix.ra"].shape == (2, 10, 10)
+    model = LadusunForCausalLM(cfg).float()
+    model.load_weights(w.items())
+    rec, att, lat, bor = (l.mixer for l in model.layers)
+    # recurrence: y | x rows of one product, taps turned so that the last row is the current token's, both gate maps side by side per block
+    assert torch.equal(rec.in_proj.weight[:20], w["l0.mix.y"]) and torch.equal(rec.in_proj.bias[20:], w["l0.mix.x.b"])
+    assert torch.equal(rec.conv_w, w["l0.mix.conv"].t()) and torch.equal(rec.conv_w[2], w["l0.mix.conv"][:, 2])
+    assert torch.equal(rec.gate_w[1, :, :10], w["l0.mix.ra"][1].t()) and torch.equal(rec.gate_w[0, :, 10:], w["l0.mix.ri"][0].t())
+    assert torch.equal(rec.gate_b[0], w["l0.mix.ra.b"].reshape(-1)) and torch.equal(rec.gate_b[1], w["l0.mix.ri.b"].reshape(-1))
+    assert torch.allclose(rec.rate, 8.0 * torch.nn.functional.softplus(w["l0.mix.lam"]), atol=1e-6)
+    # attention: q | k | v | g rows; the gate's rows have no bias
+    rows = att.in_proj.weight
+    assert rows.shape[0] == 40 + 20 + 12 + 4 and torch.equal(rows[40:60], w["l1.mix.k"]) and torch.equal(rows[60:72], w["l1.mix.v"]) and torch.equal(rows[72:], w["l1.mix.g"])
+    assert torch.equal(att.in_proj.bias[:40], w["l1.mix.q.b"]) and torch.equal(att.in_proj.bias[60:72], w["l1.mix.v.b"]) and not att.in_proj.bias[72:].any()
+    assert torch.equal(att.o_proj.bias, w["l1.mix.o.b"]) and att.sink_score == 0.0 and att.softcap == 12.0 and att.interleaved
+    assert bor.in_proj.weight.shape[0] == 20 + 2 and torch.equal(bor.in_proj.weight[:20], w["l3.mix.q"]) and bor.borrows and bor.k_name == (1, "k")
+    # latent attention: q | dkv | g rows; the maps widened to the cache row with an identity block for the rotated columns
+    rows = lat.in_proj.weight
+    assert rows.shape[0] == 42 + 13 + 3 and torch.equal(rows[42:55], w["l2.mix.dkv"]) and torch.equal(rows[55:], w["l2.mix.g"])
+    assert lat.row == 32 and torch.equal(lat.uk[1, :8, :7], w["l2.mix.uk"].view(3, 8, 7)[1]) and torch.equal(lat.uk[2, 8:, 7:13], torch.eye(6))
+    assert not lat.uk[:, :8, 7:].any() and not lat.uk[:, 8:, :7].any() and not lat.uk[:, :, 13:].any()
+    assert torch.equal(lat.uv[0, :7], w["l2.mix.uv"].view(3, 5, 7)[0].t()) and not lat.uv[:, 7:].any() and torch.equal(lat.kv_norm, w["l2.mix.dkv.norm"])
+    # feed-forwards, stream weights
+    moe, dense = model.layers[2].mlp, model.layers[1].mlp
+    assert torch.equal(moe.w_gu[2, 18:], w["l2.mlp.e2.up"]) and torch.equal(moe.w_d[0], w["l2.mlp.e0.down"]) and torch.equal(moe.router, w["l2.mlp.router"])
+    assert (moe.groups, moe.keep, moe.top, model.layers[3].mlp.groups) == (3, 1, 2, 0)
+    assert torch.equal(dense.up.bias, w["l1.mlp.up.b"]) and torch.equal(dense.down.weight, w["l1.mlp.down"])
+    hc = model.layers[1].hc2
+    assert torch.equal(hc.mix, w["l1.hc2.mix"]) and torch.equal(hc.w_in, w["l1.hc2.in"]) and torch.equal(hc.ls, w["l1.ls2"]) and torch.equal(hc.norm, w["l1.norm2"])
+    assert not hasattr(model.layers[0], "hc2")
+    assert model.latent_ranks() == {(1, "k"): 20, (1, "v"): 12, 2: 32}
+    assert model.state_shapes() == {((0, "mix"), "S"): (20,), ((0, "mix"), "conv"): (2, 20)}
+    with pytest.raises(KeyError):
+        model.load_weights([(k, v) for k, v in w.items() if k != "l1.mix.k.b"])
+    with pytest.raises(KeyError):
+        model.load_weights(list(w.items()) + [("l3.mix.k", torch.zeros(20, 36))])
+
+
+def test_frequency_tables_of_both_scalings():
+    from nano_vllm_x_amd.layers.rotary_embedding import rotary_frequencies
+    for dims, base, sc in ((8, 300.0, BANDS), (64, 5e4, {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 512}), (6, 41.0, None),
+                           (2, 10.0, {"factor": 2.0, "low": 2.0, "high": 3.0, "original": 7})):
+        want, mag = lo.banded_frequencies(dims, base, sc) if sc else (lo.plain_frequencies(dims, base), 1.0)
+        got, got_mag = rotary_frequencies(dims, base, sc)
+        assert got_mag == mag == 1.0 and torch.allclose(got, want, rtol=1e-13, atol=0)
+    f = rotary_frequencies(8, 300.0, BANDS)[0]
+    plain = lo.plain_frequencies(8, 300.0)
+    assert f[0] == plain[0] and abs(f[3] - plain[3] / 3.0) < 1e-15 and plain[1] / 3.0 < f[1] < plain[1] and plain[2] / 3.0 < f[2] < plain[2]
+    for dims, base, sc in ((6, 200.0, RAMP), (32, 2.5e5, {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}),
+                           (4, 900.0, {"factor": 8.0, "original": 16, "fast": 2.0, "slow": 0.25}), (2, 50.0, {"factor": 1.5, "original": 9, "fast": 3.0, "slow": 2.0})):
+        want, mag = lo.ramped_frequencies(dims, base, sc)
+        got, got_mag = rotary_frequencies(dims, base, sc)
+        assert abs(got_mag - mag) < 1e-15 and mag == 0.1 * math.log(sc["factor"]) + 1.0 and torch.allclose(got, want, rtol=1e-13, atol=0)
+
+
+def test_restatement_is_causal_and_its_parts_have_the_stated_form():
+    from nano_vllm_x_amd.ladusun import LadusunConfig, random_checkpoint
+    cfg = LadusunConfig.from_dict(CFG)
+    w = dict(random_checkpoint(cfg, 1))
+    toks = torch.randint(0, 53, (12,), generator=torch.Generator().manual_seed(0)).tolist()
+    sums = []
+    full = lo.forward(CFG, w, toks, sums)
+    assert len(sums) == 4 and sums[0].shape == (12, 36)
+    assert torch.allclose(lo.forward(CFG, w, toks[:7]), full[:7], atol=1e-12)
+    assert (lo.forward(CFG, w, [(toks[0] + 1) % 53] + toks[1:])[-1] - full[-1]).abs().max() > 1e-6
+    g = torch.Generator().manual_seed(2)
+    q, k, v = torch.randn(5, 4, generator=g).double(), torch.randn(5, 4, generator=g).double(), torch.randn(5, 3, generator=g).double()
+    pos = torch.arange(5)
+    # the silent term: a first token whose score is 0 gets half of its value; the weights of a row add up to less than one
+    o = lo.sink_softmax_readout(torch.zeros(1, 4).double(), k[:1], v[:1], pos[:1], pos[:1], 0.5)
+    assert torch.allclose(o, 0.5 * v[:1])
+    ones = lo.sink_softmax_readout(q, k, torch.ones(5, 1).double(), pos, pos, 0.5, cap=3.0)
+    assert (ones < 1.0).all() and (ones > 0.0).all()
+    assert torch.allclose(lo.sink_softmax_readout(q, k, torch.ones(5, 1).double(), pos, pos, 0.5, sink=None), torch.ones(5, 1).double())
+    # the cap bounds the scores: with a huge scale a visible key's weight is at most e^cap / (1 + e^cap)
+    big = lo.sink_softmax_readout(q[:1], k[:1], torch.ones(1, 1).double(), pos[:1], pos[:1], 1e6 * float(torch.sign(q[0] @ k[0])), cap=2.0)
+    assert torch.allclose(big, torch.tensor([[math.exp(2.0) / (1.0 + math.exp(2.0))]]).double())
+    # neighbours are paired: turning by a quarter of a circle sends (a, b) to (-b, a)
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0, 5.0]]).double()
+    turned = lo.turn_pairs(x, torch.tensor([1]), torch.tensor([math.pi / 2, math.pi]).double())
+    assert torch.allclose(turned, torch.tensor([[-2.0, 1.0, -3.0, -4.0, 5.0]]).double(), atol=1e-12)
+    # the recurrence: a gate far below zero keeps the state, the first token enters an empty state like every other
+    u = torch.randn(6, 3, generator=g).double()
+    s = lo.gated_recurrence(u, torch.full((6, 3), -50.0).double(), torch.zeros(6, 3).double(), torch.zeros(3).double())
+    assert s.abs().max() < 1e-8
+    r0 = torch.zeros(6, 3).double()
+    s = lo.gated_recurrence(u, r0, r0, torch.zeros(3).double())
+    a = math.exp(-8.0 * 0.5 * math.log(2.0))
+    assert torch.allclose(s[0], math.sqrt(1 - a * a) * 0.5 * u[0]) and torch.allclose(s[1], a * s[0] + math.sqrt(1 - a * a) * 0.5 * u[1])
+    # the convolution's last column is the current token's
+    taps = torch.tensor([[0.0, 0.0, 2.0]]).double()
+    assert torch.allclose(lo.causal_conv(u[:, :1], taps, torch.tensor([1.0]).double()), 2.0 * u[:, :1] + 1.0)
+    taps = torch.tensor([[3.0, 0.0, 0.0]]).double()
+    assert torch.allclose(lo.causal_conv(u[:, :1], taps, torch.zeros(1).double())[2:], 3.0 * u[:4, :1])
+    # the router: only experts of the best groups, weights that add up to one
+    z = torch.tensor([[0.0, 5.0, 4.0, 4.5, 1.0, 3.0]]).double()
+    ids, wts = lo.route_logits(z, {"experts": 6, "top": 2, "groups": {"count": 3, "keep": 1}})
+    assert sorted(ids[0].tolist()) == [0, 1] and abs(wts.sum().item() - 1.0) < 1e-12
+    ids, _ = lo.route_logits(z, {"experts": 6, "top": 2, "groups": {"count": 3, "keep": 2}})
+    assert sorted(ids[0].tolist()) == [1, 3]
+    # all streams move at once, from the old ones
+    xs = [torch.ones(1, 2).double(), 2 * torch.ones(1, 2).double()]
+    new = lo.move_streams(xs, torch.zeros(1, 2).double(), torch.tensor([[0.0, 1.0], [1.0, 0.0]]).double(), torch.zeros(2).double())
+    assert torch.equal(new[0], xs[1]) and torch.equal(new[1], xs[0])
+    new = lo.move_streams(xs, torch.ones(1, 2).double(), torch.tensor([[1.0, 10.0], [0.0, 1.0]]).double(), torch.tensor([0.5, 0.0]).double())
+    assert torch.equal(new[0], 1.5 * torch.ones(1, 2).double()) and torch.equal(new[1], 12.0 * torch.ones(1, 2).double())
+
+
+def test_configurations_of_the_device_tests_are_read_alike_by_both_sides():
+    """Every configuration the device tests use parses in the package and runs through the restatement with the package's random
+    weights (names and shapes agree)."""
+    import importlib.util
+    import os
+    spec = importlib.util.spec_from_file_location("gpu_ladusun", os.path.join(os.path.dirname(os.path.abspath(__file__)), "test_gpu_ladusun.py"))
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    for name, (layers, streams) in mod.ONE.items():
+        cfg = mod.make_cfg(layers, streams=streams)
+        out = lo.forward(cfg, mod.weights_of(cfg, 0), [1, 5, 2, 60, 0])
+        assert out.shape == (5, 61) and torch.isfinite(out).all(), name
