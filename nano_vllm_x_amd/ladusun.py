@@ -292,14 +292,21 @@ class LadusunForCausalLM(nn.Module):
     @torch.no_grad()
     def load_weights(self, weights: Iterable):
         """Checkpoint tensors under the design's names ('embed', 'l<i>.mix.q', 'l<i>.hc1.mix', 'l<i>.mlp.e<j>.up', ...) -> the fused
-        parameters."""
-        got = set()
+        parameters.  Every tensor the configuration calls for must be there, in its shape; a tensor it does not call for is left
+        out with a warning (nothing of the model reads it)."""
+        wanted, got, surplus = checkpoint_shapes(self.config), set(), []
         for name, w in weights:
+            if name not in wanted:
+                surplus.append(name)
+                continue
             self._load_one(name, w)
             got.add(name)
-        missing = [n for n in checkpoint_names(self.config) if n not in got]
+        missing = [n for n in wanted if n not in got]
         if missing:
             raise KeyError(f"checkpoint lacks {len(missing)} tensors, e.g. {missing[:4]}")
+        if surplus:
+            import warnings
+            warnings.warn(f"checkpoint holds {len(surplus)} tensors that this configuration does not use, e.g. {surplus[:4]}")
         self.pack_decode_weights()
 
     def _load_one(self, name: str, w: torch.Tensor):

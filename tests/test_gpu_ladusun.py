@@ -365,6 +365,8 @@ ONE = {
     "dense feed-forward": ([dict(REC, mlp=DENSE)], 3),
     "experts in groups": ([dict(REC, mlp=MOE)], 3),
     "experts, all of all": ([dict(REC, mlp={"kind": "moe", "expert": {"ff": 8, "limit": 0.5}, "router": {"experts": 3, "top": 3}})], 3),
+    "experts, more than the expert order holds": ([dict(REC, mlp={"kind": "moe", "expert": {"ff": 4, "limit": 2.0},
+                                                                  "router": {"experts": 70, "top": 4, "groups": {"count": 10, "keep": 3}}})], 2),
     "experts, every group kept": ([dict(REC, mlp={"kind": "moe", "expert": {"ff": 8, "limit": 3.0},
                                                   "router": {"experts": 6, "top": 2, "groups": {"count": 2, "keep": 2}}})], 3),
 }
@@ -525,9 +527,9 @@ def test_checkpoint_with_a_missing_or_misshapen_tensor_is_refused(tmp_path):
     with pytest.raises(ValueError):
         make_engine(model_dir(tmp_path, cfg, bad, name="shape"))
     bad = dict(w)
-    bad["l1.mix.k"] = torch.zeros(24, 40)
-    with pytest.raises(KeyError):
-        make_engine(model_dir(tmp_path, cfg, bad, name="extra"))
+    bad["l0.mix.q"] = w["l0.mix.q"].t().contiguous()
+    with pytest.raises(ValueError):
+        make_engine(model_dir(tmp_path, cfg, bad, name="transposed"))
 
 
 # ---- generation: the scheduler's own choices ---------------------------------------------------------------------------

@@ -93,8 +93,9 @@ def test_checkpoint_tensors_land_in_the_fused_parameters():
     assert model.state_shapes() == {((0, "mix"), "S"): (20,), ((0, "mix"), "conv"): (2, 20)}
     with pytest.raises(KeyError):
         model.load_weights([(k, v) for k, v in w.items() if k != "l1.mix.k.b"])
-    with pytest.raises(KeyError):
+    with pytest.warns(UserWarning, match="does not use"):      # a tensor that nothing reads is left out, and said so
         model.load_weights(list(w.items()) + [("l3.mix.k", torch.zeros(20, 36))])
+    assert torch.equal(bor.in_proj.weight[:20], w["l3.mix.q"])
 
 
 def test_frequency_tables_of_both_scalings():
