@@ -238,6 +238,26 @@ __global__ __launch_bounds__(256) void moe_glu_kernel(const A* __restrict__ gu, 
     }
 }
 
+// The same for 16-bit formats, eight neighbouring entries of a row per thread as one 16-byte load of each half and one store
+// (ff8 = ff / 8; rows start on 16-byte borders).
+template <typename A>
+__global__ __launch_bounds__(256) void moe_glu_vec8_kernel(const A* __restrict__ gu, A* __restrict__ y, float limit, float alpha, float shift,
+                                                          int64_t rows, int ff8) {
+    union Pack { uint4 v; A a[8]; };
+    const int64_t n = rows * ff8;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) {
+        const int64_t r = i / ff8;
+        const int64_t j = (i - r * ff8) * 8;
+        const A* row = gu + r * 16 * ff8;
+        Pack g, u, o;
+        g.v = *reinterpret_cast<const uint4*>(row + j);
+        u.v = *reinterpret_cast<const uint4*>(row + (int64_t)ff8 * 8 + j);
+#pragma unroll
+        for (int k = 0; k < 8; ++k) o.a[k] = (A)glu_act((float)g.a[k], (float)u.a[k], limit, alpha, shift);
+        *reinterpret_cast<uint4*>(y + i * 8) = o.v;
+    }
+}
+
 // out[t] = sum_k wts[t * top + k] * ys[dst[t * top + k]]   (wts == null: ones)
 template <typename A>
 __global__ __launch_bounds__(256) void moe_gather_rows_kernel(const A* __restrict__ ys, const int64_t* __restrict__ dst,
@@ -376,6 +396,17 @@ extern "C" int nvx_moe_glu(const void* gu, int fmt, float limit, float alpha, fl
     NVX_REQUIRE(fmt >= 0 && fmt <= 2 && rows >= 0 && ff > 0, NVX_EINVAL, "nvx_moe_glu: bad arguments");
     if (rows == 0) return NVX_OK;
     NVX_REQUIRE(gu && y, NVX_EINVAL, "nvx_moe_glu: null pointer");
+    if (fmt != 2 && ff % 8 == 0 && nvx_aligned16(gu) && nvx_aligned16(y)) {
+        int64_t blocks = (rows * (ff / 8) + 255) / 256;
+        if (blocks > 256 * 64) blocks = 256 * 64;
+        if (fmt == 0)
+            hipLaunchKernelGGL(moe_glu_vec8_kernel<__bf16>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const __bf16*)gu, (__bf16*)y,
+                               limit, alpha, shift, rows, (int)(ff / 8));
+        else
+            hipLaunchKernelGGL(moe_glu_vec8_kernel<_Float16>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const _Float16*)gu,
+                               (_Float16*)y, limit, alpha, shift, rows, (int)(ff / 8));
+        return nvx_check_launch("nvx_moe_glu");
+    }
     int64_t blocks = (rows * ff + 255) / 256;
     if (blocks > 256 * 64) blocks = 256 * 64;
     NVX_FMT_CALL(fmt, hipLaunchKernelGGL(moe_glu_kernel<A_>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const A_*)gu, (A_*)y, limit,

@@ -239,6 +239,22 @@ __global__ __launch_bounds__(256) void relu2_kernel(const A* __restrict__ x, A* 
     }
 }
 
+// 16-bit formats, eight entries per thread as one 16-byte load and store (n8 = n / 8)
+template <typename A>
+__global__ __launch_bounds__(256) void relu2_vec8_kernel(const A* __restrict__ x, A* __restrict__ y, int64_t n8) {
+    union Pack { uint4 v; A a[8]; };
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n8; i += (int64_t)gridDim.x * 256) {
+        Pack in, out;
+        in.v = reinterpret_cast<const uint4*>(x)[i];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const float v = fmaxf((float)in.a[k], 0.f);
+            out.a[k] = (A)(v * v);
+        }
+        reinterpret_cast<uint4*>(y)[i] = out.v;
+    }
+}
+
 // ---- minGRU ---------------------------------------------------------------------------------------------------------
 // zxg[t] = [ z pre-activation | candidate pre-activation u | output-gate pre-activation g ], `width` each.
 //   z = sigmoid(.),  cand = u + 1/2 (u >= 0) or sigmoid(u) (u < 0),  S <- (1 - z) S + z cand,  out = S * silu(g)
@@ -610,6 +626,16 @@ extern "C" int nvx_relu2(const void* x, void* y, int fmt, int64_t n, nvx_stream_
     NVX_REQUIRE(fmt >= 0 && fmt <= 2 && n >= 0, NVX_EINVAL, "nvx_relu2: bad arguments");
     if (n == 0) return NVX_OK;
     NVX_REQUIRE(x && y, NVX_EINVAL, "nvx_relu2: null pointer");
+    if (fmt != 2 && n % 8 == 0 && nvx_aligned16(x) && nvx_aligned16(y)) {
+        int64_t blocks = (n / 8 + 255) / 256;
+        if (blocks > 256 * 64) blocks = 256 * 64;
+        if (fmt == 0)
+            hipLaunchKernelGGL(relu2_vec8_kernel<__bf16>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const __bf16*)x, (__bf16*)y, n / 8);
+        else
+            hipLaunchKernelGGL(relu2_vec8_kernel<_Float16>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const _Float16*)x, (_Float16*)y,
+                               n / 8);
+        return nvx_check_launch("nvx_relu2");
+    }
     int64_t blocks = (n + 255) / 256;
     if (blocks > 256 * 64) blocks = 256 * 64;
     NVX_FMT_DISPATCH(fmt, hipLaunchKernelGGL(relu2_kernel<A_>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const A_*)x,

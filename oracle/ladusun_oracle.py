@@ -195,10 +195,15 @@ def route_logits(z, router):
     return ids, chosen / (chosen.sum(-1, keepdim=True) + 1e-20)
 
 
+def limited_glu(g, u, limit):
+    """The gate capped from above, the other branch clamped on both sides and shifted by one."""
+    g = torch.clamp(g, max=limit)
+    u = torch.clamp(u, -limit, limit)
+    return g * torch.sigmoid(1.702 * g) * (u + 1.0)
+
+
 def expert(h, w, p, limit):
-    g = torch.clamp(h @ w[p + "gate"].T, max=limit)
-    u = torch.clamp(h @ w[p + "up"].T, -limit, limit)
-    return (g * torch.sigmoid(1.702 * g) * (u + 1.0)) @ w[p + "down"].T
+    return limited_glu(h @ w[p + "gate"].T, h @ w[p + "up"].T, limit) @ w[p + "down"].T
 
 
 def moe_ff(h, w, p, mlp):

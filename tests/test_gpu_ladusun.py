@@ -305,7 +305,7 @@ def test_gated_recurrence_over_cuts_and_reused_slots(width, blocks):
         assert ((ref(full[0][1:])[-1] - want[0][-1]).abs()[slow] / (want[0][-1].abs()[slow] + 1e-3)).max() > 1e-3
 
 
-@pytest.mark.parametrize("experts,top,groups,keep", [(6, 3, 3, 2), (16, 4, 4, 3), (4, 1, 0, 0), (8, 3, 4, 4), (12, 6, 2, 1), (5, 5, 0, 0), (9, 2, 9, 2), (6, 2, 3, 2)])
+@pytest.mark.parametrize("experts,top,groups,keep", [(6, 3, 3, 2), (20, 5, 4, 3), (4, 1, 0, 0), (8, 3, 4, 4), (12, 6, 2, 1), (5, 5, 0, 0), (9, 2, 9, 2), (6, 2, 3, 2)])
 def test_softmax_router_with_groups(experts, top, groups, keep):
     from nano_vllm_x_amd import ops
     g = torch.Generator().manual_seed(experts)
@@ -321,6 +321,30 @@ def test_softmax_router_with_groups(experts, top, groups, keep):
     if groups and keep < min(top, groups):       # the groups matter: without them other experts are chosen somewhere
         free, _ = lo.route_logits(z.double(), {"experts": experts, "top": top})
         assert not torch.equal(free.sort(1).values, want_order.values)
+
+
+@pytest.mark.parametrize("fmt", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,ff", [(37, 64), (5, 12), (1, 8), (300, 1536), (3, 7)])
+def test_limited_gate_times_shifted_branch(fmt, rows, ff):
+    """Rows of gate | up: sizes that take the 16-byte path in 16-bit formats and sizes that do not; values beyond the limit on both sides."""
+    from nano_vllm_x_amd import ops
+    g = torch.Generator().manual_seed(rows + ff)
+    gu = (torch.randn(rows, 2 * ff, generator=g) * 2.0).to(fmt)
+    want = lo.limited_glu(gu[:, :ff].double(), gu[:, ff:].double(), 1.5)
+    got = ops.moe_glu(gu.cuda(), 1.5, 1.702, 1.0)
+    assert got.dtype == fmt and got.shape == (rows, ff)
+    close(got.float().cpu(), want, 1e-5 if fmt == torch.float32 else 1e-2 if fmt == torch.bfloat16 else 2e-3, f"{rows} x {ff}")
+
+
+@pytest.mark.parametrize("fmt", [torch.float32, torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("shape", [(37, 64), (5, 12), (1, 8), (300, 1536), (3, 7)])
+def test_squared_relu(fmt, shape):
+    from nano_vllm_x_amd import ops
+    x = (torch.randn(*shape, generator=torch.Generator().manual_seed(shape[1])) * 2.0).to(fmt)
+    got = ops.relu2(x.cuda())
+    assert got.dtype == fmt and got.shape == shape
+    want = torch.relu(x.double()) ** 2
+    assert torch.equal(got.cpu(), want.to(fmt)) or fmt == torch.float32 and torch.allclose(got.cpu().double(), want, rtol=1e-6)
 
 
 @pytest.mark.parametrize("experts,top,groups,keep", [(6, 3, 3, 2), (3, 3, 0, 0), (4, 1, 2, 1)])
