@@ -519,13 +519,15 @@ def test_bfloat16_stays_within_rounding(tmp_path):
 
 
 def test_bfloat16_with_heads_for_the_matrix_cores(tmp_path):
-    """Head sizes the tile kernels are built for (keys 64, values 128; a latent row of 96), prompts long enough to take them, in
+    """Head sizes the tile kernels are built for (keys 64, values 128; latent rows of 96 and of 320), prompts long enough to take them, in
     bfloat16: whole prompts against portions and single tokens, and both against the restatement within rounding."""
     att = {"type": "attention", "mixer": {"heads": 4, "kv_heads": 2, "dim": 64, "vdim": 128, "scale": 0.125, "softcap": 20.0,
                                           "rot": {"dims": 32, "base": 1e4, "scaling": {"factor": 2.0, "low": 1.0, "high": 4.0, "original": 32}}}, "mlp": DENSE}
     lat = {"type": "latent_attention", "mixer": {"heads": 4, "dim": 32, "rot_dim": 16, "vdim": 48, "kv_rank": 80, "scale": 0.14,
                                                  "rot": {"dims": 16, "base": 1e4, "scaling": RAMP}}, "mlp": MOE}
-    cfg = make_cfg([att, lat, borrowing(att, 0)], width=128, vocab=97, emb=8.0)
+    wide = {"type": "latent_attention", "mixer": {"heads": 2, "dim": 16, "rot_dim": 16, "vdim": 32, "kv_rank": 300, "scale": 0.17,
+                                                  "rot": {"dims": 16, "base": 500.0}}, "mlp": None}          # a cache row of 320
+    cfg = make_cfg([att, lat, borrowing(att, 0), wide], width=128, vocab=97, emb=8.0)
     w = weights_of(cfg, 3)
     eng = make_engine(model_dir(tmp_path, cfg, w), dtype="bfloat16", pool=1024)
     toks = tokens(300, 97, 9)
