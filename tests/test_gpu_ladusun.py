@@ -472,6 +472,75 @@ def test_first_tokens_and_page_borders_in_prompts_and_decoding(tmp_path):
     eng.shutdown()
 
 
+def drawn_configuration(rnd):
+    """A configuration drawn at random: 2 to 6 layers of any kind in any order, borrowed keys from any earlier attention layer, sizes
+    from small and odd to those the matrix-core kernels take, any feed-forward or none, with or without streams."""
+    def mlp():
+        kind = rnd.choice(["dense", "moe", "moe", None])
+        if kind is None:
+            return None
+        if kind == "dense":
+            return {"kind": "dense", "ff": rnd.choice([24, 50, 128])}
+        count, per = rnd.choice([1, 2, 4]), rnd.choice([1, 2, 3])
+        keep = rnd.randint(1, count)
+        router = {"experts": count * per, "top": rnd.randint(1, min(keep * per, 4))}
+        if rnd.random() < 0.8:
+            router["groups"] = {"count": count, "keep": keep}
+        return {"kind": "moe", "expert": {"ff": rnd.choice([8, 20, 32]), "limit": rnd.choice([0.7, 2.0, 9.0])}, "router": router}
+
+    layers, lenders = [], []
+    for i in range(rnd.randint(2, 6)):
+        kind = rnd.choice(["attention", "latent_attention", "rglru"])
+        if kind == "attention" and lenders and rnd.random() < 0.4:
+            src = rnd.choice(lenders)
+            m = dict(layers[src]["mixer"], kv_from=src, scale=rnd.choice([0.1, 0.3]))
+        elif kind == "attention":
+            kvh = rnd.choice([1, 2, 3])
+            dim, vdim = rnd.choice([6, 16, 64, 40]), rnd.choice([4, 24, 64, 128])
+            rot = {"dims": rnd.choice([dim, dim // 2 - dim // 2 % 2, 2]), "base": rnd.choice([50.0, 1e4, 1e6])}
+            if rnd.random() < 0.7:
+                rot["scaling"] = {"factor": rnd.choice([2.0, 8.0]), "low": rnd.choice([0.5, 2.0]), "high": rnd.choice([3.0, 8.0]), "original": rnd.choice([16, 100, 1000])}
+            m = {"heads": kvh * rnd.choice([1, 2, 4]), "kv_heads": kvh, "dim": dim, "vdim": vdim, "scale": dim ** -0.5 * rnd.choice([1.0, 2.0]), "rot": rot}
+            if rnd.random() < 0.7:
+                m["softcap"] = rnd.choice([3.0, 25.0])
+            lenders.append(i)
+        elif kind == "latent_attention":
+            rd, dim = rnd.choice([2, 8, 16]), rnd.choice([4, 16, 48])
+            rot = {"dims": rd, "base": rnd.choice([100.0, 2e5])}
+            if rnd.random() < 0.7:
+                rot["scaling"] = {"factor": rnd.choice([1.5, 4.0, 16.0]), "original": rnd.choice([32, 300, 2000]), "fast": rnd.choice([4.0, 16.0]), "slow": rnd.choice([0.5, 2.0])}
+            m = {"heads": rnd.choice([1, 2, 5]), "dim": dim, "rot_dim": rd, "vdim": rnd.choice([6, 32, 80]), "kv_rank": rnd.choice([5, 24, 90, 250]),
+                 "scale": (dim + rd) ** -0.5, "rot": rot}
+        else:
+            blocks = rnd.choice([1, 2, 3, 8])
+            m = {"width": blocks * rnd.choice([1, 5, 16]), "blocks": blocks, "conv": rnd.choice([1, 2, 3, 5])}
+        layers.append({"type": kind, "mixer": m, "mlp": mlp()})
+    return make_cfg(layers, width=rnd.choice([24, 50, 96, 160]), vocab=rnd.choice([37, 130, 301]), eps=rnd.choice([1e-5, 1e-6]),
+                    emb=rnd.choice([1.0, 5.0, 12.0]), streams=rnd.choice([None, 1, 2, 3, 4, 6]))
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Whole, in portions of drawn sizes with single tokens at the end, and two requests of unequal length side by side."""
+    import random
+    rnd = random.Random(seed)
+    cfg = drawn_configuration(rnd)
+    w = weights_of(cfg, seed)
+    eng = make_engine(model_dir(tmp_path, cfg, w), pool=512)
+    n = rnd.choice([70, 131, 200])
+    toks, other = tokens(n, cfg["vocab"], seed), tokens(45, cfg["vocab"], seed + 100)
+    want, want_other = forward(cfg, w, toks), forward(cfg, w, other)
+    what = json.dumps(cfg)
+    close(replay(eng, {"a": toks}, [[("a", n)]])["a"], want, F32_TOL, "whole: " + what)
+    cuts = cuts_of(n - 9, [rnd.choice([2, 3, 17, 64, 65]) for _ in range(5)]) + [1] * 9
+    close(replay(eng, {"b": toks}, [[("b", c)] for c in cuts])["b"], want, F32_TOL, "cut: " + what)
+    sched = [[("c", 30), ("d", 2)], [("c", 1), ("d", 40)]] + [[("c", 1), ("d", 1)]] * 3 + [[("c", n - 34)]]
+    got = replay(eng, {"c": toks, "d": other}, sched)
+    close(got["c"], want, F32_TOL, "side by side: " + what)
+    close(got["d"], want_other, F32_TOL, "side by side, the shorter one: " + what)
+    eng.shutdown()
+
+
 # ---- the whole stack ------------------------------------------------------------------------------------------------------
 def test_batches_of_unequal_requests_in_a_small_pool(tmp_path):
     """Four live requests at most in a pool smaller than the sum of all: portions beside single tokens, a request that
