@@ -1298,14 +1298,17 @@ def moe_order(idx, n_exp: int):
     return dst, counts
 
 
-def moe_scatter_rows(h, wts, dst):
-    """xs[dst[r]] = wts[r] * h[r // top] for every (token, choice) pair r (dst: int64 (T, top), a permutation; wts None: ones)."""
+def moe_scatter_rows(h, wts, dst, spare_rows: int = 0):
+    """xs[dst[r]] = wts[r] * h[r // top] for every (token, choice) pair r (dst: int64 (T, top), a permutation; wts None: ones).
+    `spare_rows` more rows of zeros follow the T * top rows (room for products that run a little past the last pair)."""
     _dev(h, wts, dst)
     t, top = dst.shape
     _need(h.dim() == 2 and h.shape[0] == t and h.stride(1) == 1, "moe_scatter_rows: shapes")
     _need(wts is None or (wts.dtype == F32 and wts.is_contiguous() and wts.shape == dst.shape), "moe_scatter_rows: wts must be float32 (T, top)")
     _need(dst.dtype == torch.int64 and dst.is_contiguous(), "moe_scatter_rows: dst must be int64 (T, top)")
-    xs = torch.empty((t * top, h.shape[1]), dtype=h.dtype, device=h.device)
+    xs = torch.empty((t * top + spare_rows, h.shape[1]), dtype=h.dtype, device=h.device)
+    if spare_rows:
+        xs[t * top:].zero_()
     lib = _lib.load()
     _lib.check(lib.nvx_moe_scatter_rows(_ptr(h), h.stride(0), _fmt(h), _ptr(wts), _ptr(dst), top, _ptr(xs), t, h.shape[1], _stream()),
                "nvx_moe_scatter_rows")
@@ -1325,11 +1328,11 @@ def moe_glu(gu, limit: float, alpha: float, shift: float = 1.0):
 
 
 def moe_gather_rows(ys, dst, wts=None):
-    """out[t] = sum_k wts[t][k] * ys[dst[t][k]] (wts None: ones)."""
+    """out[t] = sum_k wts[t][k] * ys[dst[t][k]] (wts None: ones); ys may have spare rows behind the T * top that dst names."""
     _dev(ys, dst, wts)
     _need(wts is None or (wts.dtype == F32 and wts.is_contiguous() and wts.shape == dst.shape), "moe_gather_rows: wts must be float32 (T, top)")
     t, top = dst.shape
-    _need(ys.dim() == 2 and ys.is_contiguous() and ys.shape[0] == t * top and dst.dtype == torch.int64 and dst.is_contiguous(), "moe_gather_rows: shapes")
+    _need(ys.dim() == 2 and ys.is_contiguous() and ys.shape[0] >= t * top and dst.dtype == torch.int64 and dst.is_contiguous(), "moe_gather_rows: shapes")
     out = torch.empty((t, ys.shape[1]), dtype=ys.dtype, device=ys.device)
     lib = _lib.load()
     _lib.check(lib.nvx_moe_gather_rows(_ptr(ys), _fmt(ys), _ptr(dst), _ptr(wts), top, _ptr(out), t, ys.shape[1], _stream()), "nvx_moe_gather_rows")
